@@ -236,7 +236,7 @@ def _declare(l):
 # ---- the sequence-mixer library (include/exl3_mix.h, csrc/mix_*.hip) -------------------------------------------------------------
 MIX_LIB_PATH = os.path.join(_HERE, "libexl3_mix.so")
 MIX_HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "exl3_mix.h")
-MIX_ABI_VERSION = 2
+MIX_ABI_VERSION = 3
 _mix = None
 
 
@@ -326,3 +326,15 @@ def _declare_mix(l):
     sig("exl3_mix_latent_decode_mfma_scratch", i32, i32, i32, i32, ctypes.POINTER(i64))
     sig("exl3_mix_latent_decode_mfma", vp, i64, i64, vp, i64, i64, vp, i64, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp)
     sig("exl3_mix_latent_decode", vp, i64, i64, vp, i64, i64, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp)
+    sig("exl3_mix_attn_prefill_ex", vp, i32, vp, i64, vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, f32, i32, i32, i32, vp)
+    sig("exl3_mix_attn_prefill_mfma_ex", vp, i32, vp, i64, vp, i64, vp, i64, vp, i64, vp, vp, i32, i32, i32, i32, i32, i32, i32, f32, f32, i32, i32, vp)
+    sig("exl3_mix_attn_decode_ex", vp, i32, vp, i64, vp, vp, vp, i64, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, f32, i32, i32, i32, vp)
+    sig("exl3_mix_qk_prep", vp, i64, vp, i64, vp, i64, vp, vp, vp, i32, f32, i32, f32, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_diff_combine", vp, vp, f32, f32, f32, vp, i64, i32, i32, i32, i32, vp)
+    sig("exl3_mix_residual_rms", vp, vp, i64, i32, vp, f32, vp, i64, vp, i32, vp, vp, vp, vp, i32, i32, i32, vp)
+    sig("exl3_mix_canon", vp, i64, vp, i64, vp, i32, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp)
+    sig("exl3_mix_topk_grouped", vp, vp, vp, vp, vp, i32, f32, i32, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_moe_up_act", vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_moe_expert_major_plain", vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_moe_down_id", vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_moe_combine_id", vp, vp, vp, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp)

@@ -6,17 +6,18 @@
 // One workgroup of AT_WAVES waves per (row, query head).  Keys kb + j * k_step, values vb + j * v_step, j < count: wave w takes the 64-key chunks
 // w, w + AT_WAVES, ... (one key per lane, its row read in 16-byte pieces when the layout allows), keeps its own running maximum, sum and
 // value accumulators (MAXV = ceil(vdim / 64) per lane), and the waves are merged through LDS at the end.  Wave 0 starts from the sink.
-// The query's first dim1 elements are read from q, the rest from q2 (dim1 = dim: one part).
+// The query's first dim1 elements are read from q, the rest from q2 (dim1 = dim: one part).  softcap > 0: score <- softcap tanh(score / softcap).
+// TO: the element type of the result (float keeps the weighted sum unrounded for a caller that combines several maps).
 #define AT_WAVES 4
 
 template <typename T> struct kvec;
 template <> struct kvec<bf16_t> { static constexpr int N = 8; };
 template <> struct kvec<float> { static constexpr int N = 4; };
 
-template <typename T, int MAXV>
-__device__ __forceinline__ void attn_row(T* __restrict__ out, const T* __restrict__ q, const T* q2, int dim1, const T* __restrict__ kb, int64_t k_step, const T* __restrict__ vb,
+template <typename T, int MAXV, typename TO = T>
+__device__ __forceinline__ void attn_row(TO* __restrict__ out, const T* __restrict__ q, const T* q2, int dim1, const T* __restrict__ kb, int64_t k_step, const T* __restrict__ vb,
                                          int64_t v_step, int count, int dim, int vdim, float scale, bool has_sink, float sink, float gate, bool k_vec,
-                                         float* smem)
+                                         float* smem, float softcap = 0.f)
 {
     float* qs = smem;                                   // [dim]
     float* ps = qs + dim;                               // [AT_WAVES][64]
@@ -52,6 +53,7 @@ __device__ __forceinline__ void attn_row(T* __restrict__ out, const T* __restric
             else
                 for (int c = 0; c < dim; ++c) d += qs[c] * to_f(kr[c]);
             s = d * scale;
+            if (softcap > 0.f) s = softcap * tanhf(s / softcap);
         }
         const float m_new = fmaxf(m, wave_max(s));          // finite: j0 < count, so lane 0 of the chunk holds a score
         const float p = (j < count) ? expf(s - m_new) : 0.f;
@@ -110,7 +112,7 @@ __device__ __forceinline__ void attn_row(T* __restrict__ out, const T* __restric
     for (int i = 0; i < MAXV; ++i)
     {
         const int c = lane + 64 * i;
-        if (c < vdim) out[c] = from_f<T>(acc[i] * f);
+        if (c < vdim) out[c] = from_f<TO>(acc[i] * f);
     }
 }
 

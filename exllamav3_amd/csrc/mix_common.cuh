@@ -60,6 +60,14 @@ __device__ __forceinline__ float glu_act_f(float g, float u, int kind, float lim
     u = fminf(fmaxf(u, -limit), limit);
     return g * sigmoid_f(1.702f * g) * (u + 1.0f);
 }
+// plain activations (EXL3_MIX_ACT_*): relu(z)^2, gelu in its tanh form, silu
+__device__ __forceinline__ float gelu_tanh_f(float z) { return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
+__device__ __forceinline__ float act_f(float v, int kind)
+{
+    if (kind == EXL3_MIX_ACT_RELU2) { const float t = fmaxf(v, 0.f); return t * t; }
+    if (kind == EXL3_MIX_ACT_GELU_TANH) return gelu_tanh_f(v);
+    return silu_f(v);
+}
 // log(sigmoid(z)) without cancellation on either side
 __device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 

@@ -43,7 +43,9 @@ __device__ __forceinline__ void dot_rows(const T* __restrict__ x, const T* __res
     if (TWO) rb = wave_sum(sb);
 }
 
-template <typename T>
+// GATED: hid = glu(Wg h, Wu h) (EXL3_MIX_GLU_*); otherwise hid = act(Wu h) (EXL3_MIX_ACT_*), wg unused.  A choice that names no stored expert
+// (idx outside 0 .. experts-1: an expert without weights, handled by the caller) is skipped.
+template <typename T, bool GATED>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(T* __restrict__ hid, const T* __restrict__ h, const T* __restrict__ wg, const T* __restrict__ wu,
                                                           const int32_t* __restrict__ idx, int experts, int ff, int width, int top, int vec, int act, float limit)
 {
@@ -51,20 +53,23 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(T* __restrict__ hid, c
     const int j = blockIdx.y * 4 + (threadIdx.x >> 6);
     if (j >= ff) return;
     const int lane = threadIdx.x & 63;
-    int e = idx[row];
-    e = e < 0 ? 0 : (e >= experts ? experts - 1 : e);
+    const int e = idx[row];
+    if (e < 0 || e >= experts) return;
     const T* x = h + (int64_t) (row / top) * width;
-    const T* g = wg + ((int64_t) e * ff + j) * width;
     const T* u = wu + ((int64_t) e * ff + j) * width;
-    float ag, au;
-    dot_rows<T, true>(x, g, u, width, vec != 0, ag, au);
-    // the two projections leave the matrix product in the activation type before the activation, like any other linear of the model
-    if (lane == 0) hid[(int64_t) row * ff + j] = from_f<T>(glu_act_f(to_f(from_f<T>(ag)), to_f(from_f<T>(au)), act, limit));
+    const T* g = GATED ? wg + ((int64_t) e * ff + j) * width : u;
+    float ag = 0.f, au;
+    if (GATED) dot_rows<T, true>(x, g, u, width, vec != 0, ag, au);
+    else       dot_rows<T, false>(x, u, u, width, vec != 0, au, ag);
+    // the projections leave the matrix product in the activation type before the activation, like any other linear of the model
+    if (lane == 0)
+        hid[(int64_t) row * ff + j] = from_f<T>(GATED ? glu_act_f(to_f(from_f<T>(ag)), to_f(from_f<T>(au)), act, limit) : act_f(to_f(from_f<T>(au)), act));
 }
 
 template <typename T>
 __global__ __launch_bounds__(256) void moe_down_kernel(T* __restrict__ y, const T* __restrict__ hid, const T* __restrict__ wd, const int32_t* __restrict__ idx,
-                                                       const float* __restrict__ wts, int experts, int ff, int width, int top, int vec)
+                                                       const float* __restrict__ wts, int experts, int ff, int width, int top, int vec,
+                                                       const T* __restrict__ h_id, const float* __restrict__ idw)
 {
     const int n = blockIdx.x;
     const int col = blockIdx.y * 4 + (threadIdx.x >> 6);
@@ -73,14 +78,15 @@ __global__ __launch_bounds__(256) void moe_down_kernel(T* __restrict__ y, const 
     float acc = 0.f;
     for (int r = 0; r < top; ++r)
     {
-        int e = idx[(int64_t) n * top + r];
-        e = e < 0 ? 0 : (e >= experts ? experts - 1 : e);
+        const int e = idx[(int64_t) n * top + r];
+        if (e < 0 || e >= experts) continue;
         const T* hr = hid + ((int64_t) n * top + r) * ff;
         const T* wr = wd + ((int64_t) e * width + col) * ff;
         float a, unused;
         dot_rows<T, false>(hr, wr, wr, ff, vec != 0, a, unused);
         acc += wts[(int64_t) n * top + r] * a;
     }
+    if (idw) acc += idw[n] * to_f(h_id[(int64_t) n * width + col]);         // experts that return their input, with the sum of their weights
     if (lane == 0) y[(int64_t) n * width + col] = from_f<T>(acc);
 }
 
@@ -91,16 +97,23 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(T* __restrict__ out, cons
         out[i] = from_f<T>(silu_f(to_f(g[i])) * to_f(u[i]));
 }
 
-// y[n] = sum_r wts[n][r] * sorted[where[n*top + r]]: the rows of the expert-sorted result back in token order, weighted.
+// y[n] = sum_r wts[n][r] * sorted[where[n*top + r]]: the rows of the expert-sorted result back in token order, weighted.  With idx, choices outside
+// 0 .. experts-1 have no row in `sorted` and are left out; with idw, y[n] += idw[n] * h_id[n] (experts that return their input).
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(T* __restrict__ y, const T* __restrict__ sorted, const int32_t* __restrict__ where,
-                                                          const float* __restrict__ wts, int top, int width)
+                                                          const float* __restrict__ wts, int top, int width, const int32_t* __restrict__ idx, int experts,
+                                                          const T* __restrict__ h_id, const float* __restrict__ idw)
 {
     const int n = blockIdx.x;
     for (int c = threadIdx.x; c < width; c += 256)
     {
         float acc = 0.f;
-        for (int r = 0; r < top; ++r) acc += wts[(int64_t) n * top + r] * to_f(sorted[(int64_t) where[(int64_t) n * top + r] * width + c]);
+        for (int r = 0; r < top; ++r)
+        {
+            if (idx) { const int e = idx[(int64_t) n * top + r]; if (e < 0 || e >= experts) continue; }
+            acc += wts[(int64_t) n * top + r] * to_f(sorted[(int64_t) where[(int64_t) n * top + r] * width + c]);
+        }
+        if (idw) acc += idw[n] * to_f(h_id[(int64_t) n * width + c]);
         y[(int64_t) n * width + c] = from_f<T>(acc);
     }
 }
@@ -132,7 +145,7 @@ __device__ __forceinline__ int em_list_rows(int* list, const int32_t* __restrict
     return cnt_s;
 }
 
-template <typename T>
+template <typename T, bool GATED>
 __global__ __launch_bounds__(256) void moe_gate_up_em_kernel(T* __restrict__ hid, const T* __restrict__ h, const T* __restrict__ wg, const T* __restrict__ wu,
                                                              const int32_t* __restrict__ idx, int n_rows, int ff, int width, int top, int act, float limit)
 {
@@ -141,8 +154,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_em_kernel(T* __restrict__ hid
     const int e = blockIdx.x, j = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int cnt = em_list_rows(em_list, idx, n_rows, e);
     if (cnt == 0 || j >= ff) return;
-    const T* g = wg + ((int64_t) e * ff + j) * width;
     const T* u = wu + ((int64_t) e * ff + j) * width;
+    const T* g = GATED ? wg + ((int64_t) e * ff + j) * width : u;
     for (int r0 = blockIdx.z * EM_ROWS; r0 < cnt; r0 += gridDim.z * EM_ROWS)      // a long list is shared by the workgroups along z
     {
         float sa[EM_ROWS], sb[EM_ROWS];
@@ -151,7 +164,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_em_kernel(T* __restrict__ hid
         for (int c = lane * VN; c < width; c += 64 * VN)
         {
             union { uint4 v; T e[VN]; } tg, tu;
-            tg.v = *(const uint4*) (g + c); tu.v = *(const uint4*) (u + c);
+            tu.v = *(const uint4*) (u + c);
+            if (GATED) tg.v = *(const uint4*) (g + c); else tg.v = tu.v;
             #pragma unroll
             for (int m = 0; m < EM_ROWS; ++m)
             {
@@ -163,7 +177,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_em_kernel(T* __restrict__ hid
                     for (int q = 0; q < VN; ++q)
                     {
                         const float xv = to_f(tx.e[q]);
-                        sa[m] += xv * to_f(tg.e[q]); sb[m] += xv * to_f(tu.e[q]);
+                        if (GATED) sa[m] += xv * to_f(tg.e[q]);
+                        sb[m] += xv * to_f(tu.e[q]);
                     }
                 }
             }
@@ -173,8 +188,9 @@ __global__ __launch_bounds__(256) void moe_gate_up_em_kernel(T* __restrict__ hid
         {
             if (r0 + m < cnt)
             {
-                const float ag = wave_sum(sa[m]), au = wave_sum(sb[m]);
-                if (lane == 0) hid[(int64_t) em_list[r0 + m] * ff + j] = from_f<T>(glu_act_f(to_f(from_f<T>(ag)), to_f(from_f<T>(au)), act, limit));
+                const float ag = GATED ? wave_sum(sa[m]) : 0.f, au = wave_sum(sb[m]);
+                if (lane == 0)
+                    hid[(int64_t) em_list[r0 + m] * ff + j] = from_f<T>(GATED ? glu_act_f(to_f(from_f<T>(ag)), to_f(from_f<T>(au)), act, limit) : act_f(to_f(from_f<T>(au)), act));
             }
         }
     }
@@ -224,10 +240,12 @@ __global__ __launch_bounds__(256) void moe_down_em_kernel(T* __restrict__ per, c
     }
 }
 
-extern "C" int exl3_mix_moe_expert_major_act(void* per, void* hid, const void* h, const void* wg, const void* wu, const void* wd, const int32_t* idx,
-                                             int n, int top, int experts, int ff, int width, int act, float limit, int dtype, void* stream)
+static int moe_expert_major(void* per, void* hid, const void* h, const void* wg, const void* wu, const void* wd, const int32_t* idx,
+                            int n, int top, int experts, int ff, int width, bool gated, int act, float limit, int dtype, void* stream)
 {
-    MIX_CHECK(act == EXL3_MIX_GLU_SILU || act == EXL3_MIX_GLU_CLAMPED_SWISH, "mix_moe_expert_major: unknown activation %d", act);
+    if (gated) MIX_CHECK(act == EXL3_MIX_GLU_SILU || act == EXL3_MIX_GLU_CLAMPED_SWISH, "mix_moe_expert_major: unknown gated activation %d", act);
+    else       MIX_CHECK(act >= EXL3_MIX_ACT_RELU2 && act <= EXL3_MIX_ACT_SILU, "mix_moe_expert_major: unknown activation %d", act);
+    if (!gated) wg = wu;
     MIX_CHECK(per && hid && h && wg && wu && wd && idx && n >= 0 && top > 0 && experts > 0 && ff > 0 && width > 0, "mix_moe_expert_major: bad arguments");
     const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
     MIX_CHECK(width % vn == 0 && ff % vn == 0 && (uintptr_t) h % 16 == 0 && (uintptr_t) wg % 16 == 0 && (uintptr_t) wu % 16 == 0 && (uintptr_t) wd % 16 == 0 &&
@@ -237,12 +255,28 @@ extern "C" int exl3_mix_moe_expert_major_act(void* per, void* hid, const void* h
     const int n_rows = n * top;
     const size_t sm = (size_t) n_rows * sizeof(int);
     const int gz = (n_rows + 2 * EM_ROWS - 1) / (2 * EM_ROWS);          // enough workgroups along z that a list of all rows is walked in two turns
-    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_gate_up_em_kernel<T>, dim3(experts, (ff + 3) / 4, gz), dim3(256), sm, (hipStream_t) stream, (T*) hid, (const T*) h,
-                                             (const T*) wg, (const T*) wu, idx, n_rows, ff, width, top, act, limit));
+    if (gated)
+        MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((moe_gate_up_em_kernel<T, true>), dim3(experts, (ff + 3) / 4, gz), dim3(256), sm, (hipStream_t) stream, (T*) hid, (const T*) h,
+                                                 (const T*) wg, (const T*) wu, idx, n_rows, ff, width, top, act, limit));
+    else
+        MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((moe_gate_up_em_kernel<T, false>), dim3(experts, (ff + 3) / 4, gz), dim3(256), sm, (hipStream_t) stream, (T*) hid, (const T*) h,
+                                                 (const T*) wg, (const T*) wu, idx, n_rows, ff, width, top, act, limit));
     if (int rc = mix_check_launch("mix_moe_expert_major (gate, up)")) return rc;
     MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_down_em_kernel<T>, dim3(experts, (width + 3) / 4, gz), dim3(256), sm, (hipStream_t) stream, (T*) per, (const T*) hid,
                                              (const T*) wd, idx, n_rows, ff, width));
     return mix_check_launch("mix_moe_expert_major (down)");
+}
+
+extern "C" int exl3_mix_moe_expert_major_act(void* per, void* hid, const void* h, const void* wg, const void* wu, const void* wd, const int32_t* idx,
+                                             int n, int top, int experts, int ff, int width, int act, float limit, int dtype, void* stream)
+{
+    return moe_expert_major(per, hid, h, wg, wu, wd, idx, n, top, experts, ff, width, true, act, limit, dtype, stream);
+}
+
+extern "C" int exl3_mix_moe_expert_major_plain(void* per, void* hid, const void* h, const void* wu, const void* wd, const int32_t* idx,
+                                               int n, int top, int experts, int ff, int width, int act, int dtype, void* stream)
+{
+    return moe_expert_major(per, hid, h, nullptr, wu, wd, idx, n, top, experts, ff, width, false, act, 0.f, dtype, stream);
 }
 
 extern "C" int exl3_mix_moe_expert_major(void* per, void* hid, const void* h, const void* wg, const void* wu, const void* wd, const int32_t* idx,
@@ -260,12 +294,19 @@ extern "C" int exl3_mix_silu_mul(void* out, const void* g, const void* u, int64_
     return mix_check_launch("mix_silu_mul");
 }
 
+extern "C" int exl3_mix_moe_combine_id(void* y, const void* sorted, const int32_t* where, const float* wts, const int32_t* idx, int experts, const void* h_id,
+                                       const float* idw, int n, int top, int width, int dtype, void* stream)
+{
+    MIX_CHECK(y && sorted && where && wts && n >= 0 && top > 0 && width > 0 && (!idw || h_id) && (!idx || experts > 0), "mix_moe_combine: bad arguments");
+    if (n == 0) return EXL3_MIX_OK;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_combine_kernel<T>, dim3(n), dim3(256), 0, (hipStream_t) stream, (T*) y, (const T*) sorted, where, wts, top, width,
+                                             idx, experts, (const T*) h_id, idw));
+    return mix_check_launch("mix_moe_combine");
+}
+
 extern "C" int exl3_mix_moe_combine(void* y, const void* sorted, const int32_t* where, const float* wts, int n, int top, int width, int dtype, void* stream)
 {
-    MIX_CHECK(y && sorted && where && wts && n >= 0 && top > 0 && width > 0, "mix_moe_combine: bad arguments");
-    if (n == 0) return EXL3_MIX_OK;
-    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_combine_kernel<T>, dim3(n), dim3(256), 0, (hipStream_t) stream, (T*) y, (const T*) sorted, where, wts, top, width));
-    return mix_check_launch("mix_moe_combine");
+    return exl3_mix_moe_combine_id(y, sorted, where, wts, nullptr, 0, nullptr, nullptr, n, top, width, dtype, stream);
 }
 
 extern "C" int exl3_mix_moe_gate_up_act(void* hid, const void* h, const void* wg, const void* wu, const int32_t* idx, int n, int top, int experts, int ff, int width,
@@ -276,9 +317,21 @@ extern "C" int exl3_mix_moe_gate_up_act(void* hid, const void* h, const void* wg
     if (n == 0) return EXL3_MIX_OK;
     const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
     const int vec = width % vn == 0 && (uintptr_t) h % 16 == 0 && (uintptr_t) wg % 16 == 0 && (uintptr_t) wu % 16 == 0;
-    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_gate_up_kernel<T>, dim3(n * top, (ff + 3) / 4), dim3(256), 0, (hipStream_t) stream, (T*) hid, (const T*) h,
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((moe_gate_up_kernel<T, true>), dim3(n * top, (ff + 3) / 4), dim3(256), 0, (hipStream_t) stream, (T*) hid, (const T*) h,
                                              (const T*) wg, (const T*) wu, idx, experts, ff, width, top, vec, act, limit));
     return mix_check_launch("mix_moe_gate_up");
+}
+
+extern "C" int exl3_mix_moe_up_act(void* hid, const void* h, const void* wu, const int32_t* idx, int n, int top, int experts, int ff, int width, int act, int dtype, void* stream)
+{
+    MIX_CHECK(act >= EXL3_MIX_ACT_RELU2 && act <= EXL3_MIX_ACT_SILU, "mix_moe_up_act: unknown activation %d", act);
+    MIX_CHECK(hid && h && wu && idx && n >= 0 && top > 0 && experts > 0 && ff > 0 && width > 0, "mix_moe_up_act: bad arguments");
+    if (n == 0) return EXL3_MIX_OK;
+    const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
+    const int vec = width % vn == 0 && (uintptr_t) h % 16 == 0 && (uintptr_t) wu % 16 == 0;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((moe_gate_up_kernel<T, false>), dim3(n * top, (ff + 3) / 4), dim3(256), 0, (hipStream_t) stream, (T*) hid, (const T*) h,
+                                             (const T*) wu, (const T*) wu, idx, experts, ff, width, top, vec, act, 0.f));
+    return mix_check_launch("mix_moe_up_act");
 }
 
 extern "C" int exl3_mix_moe_gate_up(void* hid, const void* h, const void* wg, const void* wu, const int32_t* idx, int n, int top, int experts, int ff, int width,
@@ -290,11 +343,17 @@ extern "C" int exl3_mix_moe_gate_up(void* hid, const void* h, const void* wg, co
 extern "C" int exl3_mix_moe_down(void* y, const void* hid, const void* wd, const int32_t* idx, const float* wts, int n, int top, int experts, int ff, int width,
                                  int dtype, void* stream)
 {
-    MIX_CHECK(y && hid && wd && idx && wts && n >= 0 && top > 0 && experts > 0 && ff > 0 && width > 0, "mix_moe_down: bad arguments");
+    return exl3_mix_moe_down_id(y, hid, wd, idx, wts, nullptr, nullptr, n, top, experts, ff, width, dtype, stream);
+}
+
+extern "C" int exl3_mix_moe_down_id(void* y, const void* hid, const void* wd, const int32_t* idx, const float* wts, const void* h_id, const float* idw,
+                                    int n, int top, int experts, int ff, int width, int dtype, void* stream)
+{
+    MIX_CHECK(y && hid && wd && idx && wts && n >= 0 && top > 0 && experts > 0 && ff > 0 && width > 0 && (!idw || h_id), "mix_moe_down: bad arguments");
     if (n == 0) return EXL3_MIX_OK;
     const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
     const int vec = ff % vn == 0 && (uintptr_t) hid % 16 == 0 && (uintptr_t) wd % 16 == 0;
     MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_down_kernel<T>, dim3(n, (width + 3) / 4), dim3(256), 0, (hipStream_t) stream, (T*) y, (const T*) hid, (const T*) wd,
-                                             idx, wts, experts, ff, width, top, vec));
+                                             idx, wts, experts, ff, width, top, vec, (const T*) h_id, idw));
     return mix_check_launch("mix_moe_down");
 }

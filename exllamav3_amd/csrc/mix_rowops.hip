@@ -8,8 +8,6 @@
 #define ROW_THREADS 256
 #define ROW_WAVES 4
 
-__device__ __forceinline__ float gelu_tanh_f(float z) { return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
-
 template <typename T>
 __global__ __launch_bounds__(ROW_THREADS) void embed_copy_kernel(float* __restrict__ x, T* __restrict__ xc, int64_t xc_ld, const T* __restrict__ table,
                                                                  const int32_t* __restrict__ tokens, int width, int vocab)
@@ -74,13 +72,6 @@ __global__ __launch_bounds__(ROW_THREADS) void dyn_tanh_rows_kernel(T* __restric
 template <typename T> struct rvec;
 template <> struct rvec<bf16_t> { static constexpr int N = 8; };
 template <> struct rvec<float> { static constexpr int N = 4; };
-
-__device__ __forceinline__ float act_f(float v, int kind)
-{
-    if (kind == 0) { const float t = fmaxf(v, 0.f); return t * t; }
-    if (kind == 1) return gelu_tanh_f(v);
-    return silu_f(v);
-}
 
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void act_kernel(T* __restrict__ out, const T* __restrict__ z, int64_t z_ld, int ff, int kind)
@@ -176,6 +167,113 @@ __global__ void topk_sigmoid_kernel(int32_t* __restrict__ idx, float* __restrict
     for (int r = 0; r < top; ++r) w[r] = w[r] * f;
 }
 
+// Router over `total` outputs of which the first `real` name stored experts and the rest experts that return their input.  One wave per row, the
+// outputs across the lanes.  Scores s: softmax over all outputs (kind 0) or independent sigmoids (kind 1).  The choice looks at c = s + correction;
+// with groups > 1 the outputs form `groups` equal groups of neighbours, a group counts as its largest c, and only the `keep` best groups can be chosen
+// from (the others count as minus infinity).  The `top` largest c are taken one after the other (ties go to the lower index); the weights are the
+// chosen s over their sum (+ 1e-20) times `scale` (normalise = 0: s * scale).  Out: idx / wts per choice -- a choice beyond the stored experts is
+// written as idx = real with weight 0 -- and idw[n] = the weights of those choices added up.
+#define TG_MAX_PER_LANE 8
+__global__ __launch_bounds__(64) void topk_grouped_kernel(int32_t* __restrict__ idx, float* __restrict__ wts, float* __restrict__ idw, const float* __restrict__ logits,
+                                                          const float* __restrict__ correction, int kind, float scale, int normalise, int groups, int keep,
+                                                          int total, int real, int top)
+{
+    __shared__ float gmax[64];
+    const int n = blockIdx.x, lane = threadIdx.x;
+    const float* l = logits + (int64_t) n * total;
+    float s[TG_MAX_PER_LANE], c[TG_MAX_PER_LANE];
+    float mx = -INFINITY;
+    #pragma unroll
+    for (int i = 0; i < TG_MAX_PER_LANE; ++i)
+    {
+        const int e = lane + 64 * i;
+        s[i] = e < total ? l[e] : -INFINITY;
+        mx = fmaxf(mx, s[i]);
+    }
+    if (kind == 0)
+    {
+        mx = wave_max(mx);
+        float den = 0.f;
+        #pragma unroll
+        for (int i = 0; i < TG_MAX_PER_LANE; ++i) { s[i] = (lane + 64 * i < total) ? expf(s[i] - mx) : 0.f; den += s[i]; }
+        den = wave_sum(den);
+        #pragma unroll
+        for (int i = 0; i < TG_MAX_PER_LANE; ++i) s[i] = s[i] / den;
+    }
+    else
+    {
+        #pragma unroll
+        for (int i = 0; i < TG_MAX_PER_LANE; ++i) s[i] = (lane + 64 * i < total) ? sigmoid_f(s[i]) : 0.f;
+    }
+    #pragma unroll
+    for (int i = 0; i < TG_MAX_PER_LANE; ++i)
+    {
+        const int e = lane + 64 * i;
+        c[i] = e < total ? (correction ? s[i] + correction[e] : s[i]) : -INFINITY;
+    }
+    if (groups > 1 && keep < groups)
+    {
+        const int per = total / groups;
+        for (int g = 0; g < groups; ++g)
+        {
+            float m = -INFINITY;
+            #pragma unroll
+            for (int i = 0; i < TG_MAX_PER_LANE; ++i) { const int e = lane + 64 * i; if (e < total && e / per == g) m = fmaxf(m, c[i]); }
+            m = wave_max(m);
+            if (lane == 0) gmax[g] = m;
+        }
+        __syncthreads();
+        unsigned long long kept = 0ull;                      // every lane picks the same groups: the `keep` largest, ties to the lower index
+        for (int r = 0; r < keep; ++r)
+        {
+            int best = -1; float bv = 0.f;
+            for (int g = 0; g < groups; ++g)
+            {
+                if ((kept >> g) & 1ull) continue;
+                if (best < 0 || gmax[g] > bv) { best = g; bv = gmax[g]; }
+            }
+            kept |= 1ull << best;
+        }
+        #pragma unroll
+        for (int i = 0; i < TG_MAX_PER_LANE; ++i) { const int e = lane + 64 * i; if (e < total && !((kept >> (e / per)) & 1ull)) c[i] = -INFINITY; }
+    }
+    float sum = 0.f, my_w = 0.f; int my_e = 0;               // lane r keeps choice r
+    unsigned taken = 0u;                                     // bit i: this lane's output lane + 64 i is chosen
+    for (int r = 0; r < top; ++r)
+    {
+        float bv = -INFINITY; int be = 0x7fffffff;
+        #pragma unroll
+        for (int i = 0; i < TG_MAX_PER_LANE; ++i)
+        {
+            const int e = lane + 64 * i;
+            if (e < total && !((taken >> i) & 1u) && (c[i] > bv || be == 0x7fffffff)) { bv = c[i]; be = e; }      // ascending e within a lane: the first of equals stays
+        }
+        #pragma unroll
+        for (int o = 32; o > 0; o >>= 1)
+        {
+            const float ov = __shfl_xor(bv, o, 64); const int oe = __shfl_xor(be, o, 64);
+            if (oe != 0x7fffffff && (be == 0x7fffffff || ov > bv || (ov == bv && oe < be))) { bv = ov; be = oe; }
+        }
+        float sv = 0.f;
+        #pragma unroll
+        for (int i = 0; i < TG_MAX_PER_LANE; ++i) if (lane + 64 * i == be) { sv = s[i]; taken |= 1u << i; }
+        sv = wave_sum(sv);
+        sum += sv;
+        if (lane == r) { my_w = sv; my_e = be; }
+    }
+    const float f = normalise ? scale / (sum + 1e-20f) : scale;
+    const bool mine = lane < top;
+    const float w = mine ? my_w * f : 0.f;
+    const bool ident = mine && my_e >= real;
+    if (mine)
+    {
+        idx[(int64_t) n * top + lane] = ident ? real : my_e;
+        wts[(int64_t) n * top + lane] = ident ? 0.f : w;
+    }
+    const float iw = wave_sum(ident ? w : 0.f);
+    if (idw && lane == 0) idw[n] = iw;
+}
+
 extern "C" int exl3_mix_embed_copy(float* x, void* xc, int64_t xc_ld, const void* table, const int32_t* tokens, int n, int width, int vocab, int dtype, void* stream)
 {
     MIX_CHECK(x && table && tokens && n >= 0 && width > 0 && vocab > 0 && (!xc || xc_ld >= width), "mix_embed_copy: bad arguments");
@@ -266,4 +364,16 @@ extern "C" int exl3_mix_topk_sigmoid(int32_t* idx, float* wts, const float* logi
     if (n == 0) return EXL3_MIX_OK;
     hipLaunchKernelGGL(topk_sigmoid_kernel, dim3((n + 63) / 64), dim3(64), 0, (hipStream_t) stream, idx, wts, logits, correction, scale, normalise, n, experts, top);
     return mix_check_launch("mix_topk_sigmoid");
+}
+
+extern "C" int exl3_mix_topk_grouped(int32_t* idx, float* wts, float* idw, const float* logits, const float* correction, int kind, float scale, int normalise,
+                                     int groups, int keep, int n, int total, int real, int top, void* stream)
+{
+    MIX_CHECK(idx && wts && logits && n >= 0 && total > 0 && real >= 0 && real <= total && (real == total || idw), "mix_topk_grouped: bad arguments");
+    MIX_CHECK(total <= 64 * TG_MAX_PER_LANE && top > 0 && top <= 64 && top <= total && (kind == 0 || kind == 1), "mix_topk_grouped: at most %d outputs, top <= 64", 64 * TG_MAX_PER_LANE);
+    MIX_CHECK(groups >= 1 && groups <= 64 && total % groups == 0 && keep >= 1 && keep <= groups && top <= keep * (total / groups),
+              "mix_topk_grouped: %d groups (keep %d) over %d outputs cannot give %d choices", groups, keep, total, top);
+    if (n == 0) return EXL3_MIX_OK;
+    hipLaunchKernelGGL(topk_grouped_kernel, dim3(n), dim3(64), 0, (hipStream_t) stream, idx, wts, idw, logits, correction, kind, scale, normalise, groups, keep, total, real, top);
+    return mix_check_launch("mix_topk_grouped");
 }

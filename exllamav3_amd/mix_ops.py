@@ -407,3 +407,203 @@ def moe_gate_up_act(hid, h, wg, wu, idx, act_kind: int, limit: float):
          and hid.shape == (n * top, ff) and hid.dtype == h.dtype == wg.dtype, "moe_gate_up: shapes")
     _i32c(idx, "idx")
     _check(_lib.mixlib().exl3_mix_moe_gate_up_act(_p(hid), _p(h), _p(wg), _p(wu), _p(idx), n, top, experts, ff, width, act_kind, limit, code(h.dtype), _stream(h)))
+
+
+# ---- several attention maps per head, chunk masks, soft-capped scores; normed and rotated queries / keys (csrc/mix_attn*.hip, mix_diffattn.hip) ---------
+MASK_WINDOW, MASK_CHUNK = 0, 1
+
+
+def qk_prep(q_view, k_view, v_view, q_norm, k_norm, freq, mag: float, interleaved: bool, eps: float, ring_k, ring_v, tok_seq, tok_pos, slots, len_after, dim: int):
+    """In place on the step's queries and keys: RMS norm per (row, head, map) with a shared weight (None: no norm), rotary positions over 2 * len(freq)
+    leading entries (None: no rotation); keys and values of the rows a sequence keeps go into the rings."""
+    n = q_view.shape[0]
+    n_slots, window, k_heads, d2 = ring_k.shape
+    v_heads, vdim = ring_v.shape[2], ring_v.shape[3]
+    _req(d2 == dim and ring_v.shape[:2] == (n_slots, window) and ring_k.is_contiguous() and ring_v.is_contiguous(), "qk_prep: ring shapes")
+    _req(q_view.shape[1] % dim == 0 and k_view.shape == (n, k_heads * dim) and v_view.shape == (n, v_heads * vdim), "qk_prep: step shapes")
+    _req(q_view.dtype == k_view.dtype == v_view.dtype == ring_k.dtype == ring_v.dtype, "qk_prep: element types")
+    for t, nm in ((tok_seq, "tok_seq"), (tok_pos, "tok_pos"), (slots, "slots"), (len_after, "len_after")):
+        _i32c(t, nm)
+    for t, nm in ((q_norm, "q_norm"), (k_norm, "k_norm")):
+        if t is not None:
+            _f32c(t, nm); _req(t.numel() == dim, f"qk_prep: {nm}")
+    if freq is not None:
+        _f32c(freq, "freq")
+    q_heads = q_view.shape[1] // dim
+    _req(tok_seq.numel() == n and tok_pos.numel() == n, "qk_prep: rows")
+    _check(_lib.mixlib().exl3_mix_qk_prep(_p(q_view), _view(q_view, q_heads * dim, "q"), _p(k_view), _view(k_view, k_heads * dim, "k"), _p(v_view),
+                                           _view(v_view, v_heads * vdim, "v"), _p(q_norm), _p(k_norm), _p(freq), 0 if freq is None else 2 * freq.numel(), mag,
+                                           1 if interleaved else 0, eps, _p(ring_k), _p(ring_v), _p(tok_seq), _p(tok_pos), _p(slots), _p(len_after),
+                                           n, q_heads, k_heads, v_heads, dim, vdim, window, code(q_view.dtype), _stream(q_view)))
+
+
+def attn_prefill_maps(out, q_view, k_view, v_view, gate_view, sink, cu, tok_seq, tok_pos, heads: int, kv_heads: int, maps: int, dim: int, vdim: int, scale: float,
+                      softcap: float, window: int, mask: int, max_rows: int = 0, mfma: bool | None = None):
+    """Prompt-step attention over the step's own keys with `maps` maps per head, a soft cap and a window or chunk mask.  out [n, heads * maps * vdim] in
+    float32 or the activation type.  mfma None: the matrix-core kernel for bfloat16 steps from ATTN_MFMA_MIN_ROWS rows."""
+    n = q_view.shape[0]
+    _req(out.is_contiguous() and out.shape == (n, heads * maps * vdim) and out.dtype in (torch.float32, q_view.dtype), "attn_prefill_maps: out")
+    _req(q_view.dtype == k_view.dtype == v_view.dtype and k_view.shape[0] == n and v_view.shape[0] == n, "attn_prefill_maps: step tensors")
+    if sink is not None:
+        _f32c(sink, "sink"); _req(sink.numel() == heads and maps == 1, "attn_prefill_maps: sink")
+    out_f32 = 1 if (out.dtype == torch.float32 and q_view.dtype != torch.float32) else 0
+    gate_ld = 0 if gate_view is None else _view(gate_view, heads, "gate")
+    if mfma is None:
+        mfma = q_view.dtype == torch.bfloat16 and max_rows >= ATTN_MFMA_MIN_ROWS and dim <= 256 and vdim <= 256 and scale > 0
+    if mfma:
+        _req(q_view.dtype == torch.bfloat16 and max_rows > 0, "attn_prefill_maps: the matrix-core kernel takes bfloat16 and the step's longest sequence")
+        _check(_lib.mixlib().exl3_mix_attn_prefill_mfma_ex(_p(out), out_f32, _p(q_view), _view(q_view, heads * maps * dim, "q"), _p(k_view), _view(k_view, kv_heads * maps * dim, "k"),
+                                                            _p(v_view), _view(v_view, kv_heads * vdim, "v"), _p(gate_view), gate_ld, _p(sink), _p(cu), cu.numel() - 1, max_rows,
+                                                            heads, kv_heads, maps, dim, vdim, scale, softcap, window, mask, _stream(out)))
+        return
+    _check(_lib.mixlib().exl3_mix_attn_prefill_ex(_p(out), out_f32, _p(q_view), _view(q_view, heads * maps * dim, "q"), _p(k_view), _view(k_view, kv_heads * maps * dim, "k"),
+                                                   _p(v_view), _view(v_view, kv_heads * vdim, "v"), _p(gate_view), gate_ld, _p(sink), _p(cu), _p(tok_seq), _p(tok_pos),
+                                                   n, heads, kv_heads, maps, dim, vdim, scale, softcap, window, mask, code(q_view.dtype), _stream(out)))
+
+
+def attn_decode_maps(out, q_view, ring_k, ring_v, gate_view, sink, slots, len_after, heads: int, maps: int, scale: float, softcap: float, mask: int):
+    """One new row per sequence against the rings (ring_k [slots, window, kv_heads * maps, dim], ring_v [slots, window, kv_heads, vdim])."""
+    n = out.shape[0]
+    n_slots, window, k_heads, dim = ring_k.shape
+    kv_heads, vdim = ring_v.shape[2], ring_v.shape[3]
+    _req(k_heads == kv_heads * maps and ring_k.is_contiguous() and ring_v.is_contiguous() and ring_k.dtype == ring_v.dtype == q_view.dtype, "attn_decode_maps: rings")
+    _req(out.is_contiguous() and out.shape == (n, heads * maps * vdim) and out.dtype in (torch.float32, q_view.dtype), "attn_decode_maps: out")
+    _req(slots.numel() == n and len_after.numel() == n and q_view.shape[0] == n, "attn_decode_maps: one row per sequence")
+    if sink is not None:
+        _f32c(sink, "sink"); _req(sink.numel() == heads and maps == 1, "attn_decode_maps: sink")
+    out_f32 = 1 if (out.dtype == torch.float32 and q_view.dtype != torch.float32) else 0
+    _check(_lib.mixlib().exl3_mix_attn_decode_ex(_p(out), out_f32, _p(q_view), _view(q_view, heads * maps * dim, "q"), _p(ring_k), _p(ring_v), _p(gate_view),
+                                                  0 if gate_view is None else _view(gate_view, heads, "gate"), _p(sink), _p(slots), _p(len_after),
+                                                  n, heads, kv_heads, maps, dim, vdim, scale, softcap, window, mask, code(q_view.dtype), _stream(out)))
+
+
+def diff_combine(out, a, lam: float, diff: float, eps: float, gate_view, heads: int, vdim: int):
+    """a [n, heads * 2 * vdim] float32 (two maps per head) -> out [n, heads * vdim] = rms_unit(a1 - lam a2) (1 - diff) sigmoid(gate)."""
+    n = out.shape[0]
+    _f32c(a, "a")
+    _req(a.shape == (n, heads * 2 * vdim) and out.is_contiguous() and out.shape == (n, heads * vdim), "diff_combine: shapes")
+    if gate_view is not None:
+        _req(gate_view.dtype == out.dtype and gate_view.shape[0] == n, "diff_combine: gate")
+    _check(_lib.mixlib().exl3_mix_diff_combine(_p(out), _p(a), lam, diff, eps, _p(gate_view), 0 if gate_view is None else _view(gate_view, heads, "gate"),
+                                                n, heads, vdim, code(out.dtype), _stream(out)))
+
+
+# ---- residual update + RMS norm + short causal input convolution (csrc/mix_canon.hip) ----------------------------------------------------------------
+def residual_rms(x, y_view, mode: int, w, eps: float, h_view, conv_w=None, ring=None, tok_seq=None, tok_pos=None, slots=None):
+    """x (float32, in place) = x | x + y | y (RES_*); h = rms_norm(x) * w, and with conv_w (steps of one row per sequence) h + its causal convolution over
+    the ring [slots, taps - 1, width] of earlier normed rows, which also receives the new one.  h_view None: the update alone."""
+    n, width = x.shape
+    _f32c(x, "x")
+    ref = y_view if y_view is not None else h_view
+    _req(ref is not None, "residual_rms: nothing to do")
+    if mode != RES_KEEP:
+        _req(y_view is not None and y_view.shape[0] == n, "residual_rms: y")
+    if h_view is not None:
+        _f32c(w, "w"); _req(w.numel() == width and h_view.shape[0] == n and h_view.dtype == ref.dtype, "residual_rms: h / w")
+    taps = 0
+    if conv_w is not None:
+        _f32c(conv_w, "conv_w"); taps = conv_w.shape[1]
+        _req(conv_w.shape[0] == width and ring is not None and ring.is_contiguous() and ring.shape[1:] == (max(taps - 1, 1), width) and ring.dtype == ref.dtype,
+             "residual_rms: convolution weights / ring")
+        for t, nm in ((tok_seq, "tok_seq"), (tok_pos, "tok_pos"), (slots, "slots")):
+            _i32c(t, nm)
+    _check(_lib.mixlib().exl3_mix_residual_rms(_p(x), _p(y_view) if mode != RES_KEEP else None, 0 if (y_view is None or mode == RES_KEEP) else _view(y_view, width, "y"), mode,
+                                                _p(w), eps, _p(h_view), 0 if h_view is None else _view(h_view, width, "h"), _p(conv_w), taps, _p(ring), _p(tok_seq), _p(tok_pos),
+                                                _p(slots), n, width, code(ref.dtype), _stream(x)))
+
+
+def canon(out, hn, conv_w, ring, tok_seq, tok_pos, slots, pos0, len_after):
+    """out = hn + causal convolution of hn over time per channel (conv_w [width, taps]) for a packed step; the ring keeps each sequence's last taps - 1 rows."""
+    n, width = hn.shape
+    taps = conv_w.shape[1]
+    _f32c(conv_w, "conv_w")
+    _req(out.shape == hn.shape and out.dtype == hn.dtype == ring.dtype and conv_w.shape[0] == width and ring.is_contiguous() and ring.shape[1:] == (max(taps - 1, 1), width),
+         "canon: shapes")
+    for t, nm in ((tok_seq, "tok_seq"), (tok_pos, "tok_pos"), (slots, "slots"), (pos0, "pos0"), (len_after, "len_after")):
+        _i32c(t, nm)
+    _check(_lib.mixlib().exl3_mix_canon(_p(out), _view(out, width, "out"), _p(hn), _view(hn, width, "hn"), _p(conv_w), taps, _p(ring), _p(tok_seq), _p(tok_pos), _p(slots),
+                                         _p(pos0), _p(len_after), n, width, code(hn.dtype), _stream(hn)))
+
+
+# ---- grouped routers, experts without weights, ungated experts (csrc/mix_rowops.hip, mix_moe.hip) ------------------------------------------------------
+ROUTE_SOFTMAX_ALL, ROUTE_SIGMOID = 0, 1
+
+
+def topk_grouped(idx, wts, idw, logits, correction, kind: int, real: int, groups: int = 1, keep: int = 1, scale: float = 1.0, normalise: bool = True):
+    """logits [n, total]: outputs >= real stand for experts that return their input (written as idx = real, weight 0, their weights summed into idw [n])."""
+    n, total = logits.shape
+    top = idx.shape[1]
+    _f32c(logits, "logits"); _f32c(wts, "wts"); _i32c(idx, "idx")
+    _req(idx.shape == wts.shape == (n, top), "topk_grouped: shapes")
+    if idw is not None:
+        _f32c(idw, "idw"); _req(idw.numel() == n, "topk_grouped: idw")
+    if correction is not None:
+        _f32c(correction, "correction"); _req(correction.numel() == total, "topk_grouped: correction")
+    _check(_lib.mixlib().exl3_mix_topk_grouped(_p(idx), _p(wts), _p(idw), _p(logits), _p(correction), kind, scale, 1 if normalise else 0, groups, keep, n, total, real, top,
+                                                _stream(logits)))
+
+
+def moe_up_act(hid, h, wu, idx, act_kind: int):
+    n, width = h.shape
+    experts, ff, w2 = wu.shape
+    top = idx.shape[1]
+    _req(h.is_contiguous() and wu.is_contiguous() and w2 == width and hid.is_contiguous() and hid.shape == (n * top, ff) and hid.dtype == h.dtype == wu.dtype, "moe_up_act: shapes")
+    _i32c(idx, "idx")
+    _check(_lib.mixlib().exl3_mix_moe_up_act(_p(hid), _p(h), _p(wu), _p(idx), n, top, experts, ff, width, act_kind, code(h.dtype), _stream(h)))
+
+
+def moe_down_id(y, hid, wd, idx, wts, h_id=None, idw=None):
+    n, width = y.shape
+    experts, w2, ff = wd.shape
+    top = idx.shape[1]
+    _req(y.is_contiguous() and hid.is_contiguous() and wd.is_contiguous() and w2 == width and hid.shape == (n * top, ff) and y.dtype == hid.dtype == wd.dtype, "moe_down: shapes")
+    _i32c(idx, "idx"); _f32c(wts, "wts")
+    if idw is not None:
+        _f32c(idw, "idw"); _req(h_id is not None and h_id.is_contiguous() and h_id.shape == y.shape and h_id.dtype == y.dtype, "moe_down: the identity share needs the input rows")
+    _check(_lib.mixlib().exl3_mix_moe_down_id(_p(y), _p(hid), _p(wd), _p(idx), _p(wts), _p(h_id) if idw is not None else None, _p(idw), n, top, experts, ff, width,
+                                               code(y.dtype), _stream(y)))
+
+
+def moe_expert_major_plain(y, h, wu, wd, idx, wts, act_kind: int, idw=None):
+    """Ungated experts of a handful to a few dozen rows, expert-major; idw: per-row weight of the experts that return their input."""
+    n, width = h.shape
+    experts, ff, _ = wu.shape
+    top = idx.shape[1]
+    _req(h.is_contiguous() and wu.is_contiguous() and wd.is_contiguous() and y.is_contiguous() and y.dtype == h.dtype == wu.dtype, "moe_expert_major_plain: layout")
+    _i32c(idx, "idx"); _f32c(wts, "wts")
+    hid = torch.empty((n * top, ff), dtype=h.dtype, device=h.device)
+    per = torch.empty((n * top, width), dtype=h.dtype, device=h.device)
+    key = (n * top, h.device)
+    if key not in _identity:
+        _identity[key] = torch.arange(n * top, dtype=torch.int32, device=h.device)
+    lib = _lib.mixlib()
+    _check(lib.exl3_mix_moe_expert_major_plain(_p(per), _p(hid), _p(h), _p(wu), _p(wd), _p(idx), n, top, experts, ff, width, act_kind, code(h.dtype), _stream(h)))
+    _check(lib.exl3_mix_moe_combine_id(_p(y), _p(per), _p(_identity[key]), _p(wts), _p(idx), experts, _p(h) if idw is not None else None, _p(idw), n, top, width,
+                                        code(h.dtype), _stream(h)))
+
+
+def moe_grouped_plain(y, h, wu, wd, idx, wts, act_kind: int, idw=None):
+    """Ungated experts of many rows: rows sorted by expert (device), one host read of the per-expert counts, per expert two vendor matrix products with the
+    activation kernel between them, and the weighted un-sort (which leaves out the choices without a stored expert and adds the identity share)."""
+    n, width = h.shape
+    experts, ff, _ = wu.shape
+    top = idx.shape[1]
+    flat = idx.reshape(-1).long()
+    order = torch.sort(flat, stable=True).indices
+    counts = torch.zeros(experts + 1, dtype=torch.int32, device=h.device).index_add_(0, flat, torch.ones_like(flat, dtype=torch.int32)).tolist()
+    where = torch.empty(n * top, dtype=torch.int32, device=h.device)
+    where[order] = torch.arange(n * top, dtype=torch.int32, device=h.device)
+    stored = sum(counts[:experts])
+    xs = h.index_select(0, order[:stored] // top)
+    out = torch.empty((n * top, width), dtype=h.dtype, device=h.device)
+    hid = torch.empty((max(stored, 1), ff), dtype=h.dtype, device=h.device)
+    lib, at = _lib.mixlib(), 0
+    for e, c in enumerate(counts[:experts]):
+        if c == 0:
+            continue
+        u = torch.nn.functional.linear(xs[at: at + c], wu[e])
+        _check(lib.exl3_mix_act(_p(hid[at: at + c]), _p(u), ff, c, ff, act_kind, code(h.dtype), _stream(h)))
+        torch.mm(hid[at: at + c], wd[e].t(), out=out[at: at + c])
+        at += c
+    _check(lib.exl3_mix_moe_combine_id(_p(y), _p(out), _p(where), _p(wts), _p(idx), experts, _p(h) if idw is not None else None, _p(idw), n, top, width,
+                                        code(h.dtype), _stream(h)))

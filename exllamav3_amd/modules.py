@@ -20,7 +20,15 @@ float32 accumulation; true float32 when the model runs in float32).
     GatedMLP                W_down glu(W_gate h, W_up h) with a gated activation (silu, or the clamped swish with its limit)
     TokenSide               per-layer token input: a gate on the residual times a slice of a second embedding, projected back and RMS-normed
     PreNormBlock            x += mixer(norm1(x)); x += ff(norm2(x)); x += side(x), each update fused with what the next consumer reads
-  SparseExperts also routes by sigmoid scores with a selection-only correction, takes either gated activation and an always-on shared expert.
+  SparseExperts also routes by sigmoid scores with a selection-only correction, takes either gated activation and an always-on shared expert;
+  with a softmax over all experts, groups of experts of which only the best are eligible, ungated experts (W_down act(W_up h)) and trailing router
+  outputs that stand for experts which return their input.
+    CanonNorm               RMS norm with a one-plus weight followed by the short causal per-channel input convolution h + conv(h), fused into the
+                            residual update that precedes it; the last taps - 1 normed rows of a sequence live in its slot
+    DifferentialAttention   grouped-query attention with two maps per head over shared values, o = a1 - lambda a2, per-head unit RMS, head-wise
+                            sigmoid gate; RMS-normed queries / keys, rotary positions (rotate-half layout, partial, YaRN), soft-capped scores, chunk
+                            (or window) mask; rings of one chunk per slot
+    CanonBlock              x += mixer(canon1(x)); x += ff(canon2(x)) over CanonNorm inputs
 
 Every sum that the model's exactness rests on (norms, scores, softmax, decays, states, the residual) is float32 inside the kernels in
 both modes; the element type only decides how matrix products and their outputs are held.
@@ -397,27 +405,39 @@ class SparseExperts:
     EXPERT_MAJOR_MIN_ROWS = 4
 
     def __init__(self, width: int, ff: int, experts: int, top: int, router: str = "softmax", router_bias: bool = True, correction: bool = False,
-                 route_scale: float = 1.0, act: str = "silu", limit: float = 0.0, shared: GatedMLP | None = None):
+                 route_scale: float = 1.0, act: str = "silu", limit: float = 0.0, shared: GatedMLP | None = None, gated: bool = True, identity: int = 0,
+                 groups: int = 1, keep_groups: int = 1):
         """router "softmax": the top logits, weights = softmax over them.  "sigmoid": scores sigmoid(z), chosen by score (+ a stored correction that the
-        weights do not see), weights = chosen scores / their sum * route_scale.  shared: an expert that every row runs, added to the routed sum."""
-        if not 0 < top <= experts:
-            raise RuntimeError(f"router: top {top} of {experts} experts")
-        if router not in ("softmax", "sigmoid"):
+        weights do not see), weights = chosen scores / their sum * route_scale.  "softmax_all": scores = softmax over all router outputs, chosen by score +
+        correction inside the `keep_groups` best of `groups` groups of neighbouring outputs, weights = chosen scores / their sum * route_scale (the grouped
+        form also serves "sigmoid" when groups > 1).  identity: the router has this many outputs beyond the stored experts; they stand for experts that return
+        their input.  gated False: experts are W_down act(W_up h) with a plain activation (ActMLP.KINDS).  shared: an expert that every row runs, added to
+        the routed sum."""
+        if not 0 < top <= experts + identity:
+            raise RuntimeError(f"router: top {top} of {experts + identity} experts")
+        if router not in ("softmax", "sigmoid", "softmax_all"):
             raise RuntimeError(f"router: unknown kind {router!r}")
+        if (identity or groups > 1) and router == "softmax":
+            raise RuntimeError("router: groups and identity experts go with the softmax_all and sigmoid routers")
+        if groups < 1 or (experts + identity) % groups or not 1 <= keep_groups <= groups or top > keep_groups * ((experts + identity) // groups):
+            raise RuntimeError(f"router: {groups} groups (keep {keep_groups}) over {experts + identity} outputs cannot give {top} choices")
         self.width, self.ff, self.experts, self.top = width, ff, experts, top
         self.router, self.has_router_bias, self.has_correction, self.route_scale = router, router_bias, correction, float(route_scale)
-        self.act_kind, self.limit, self.shared = GatedMLP.KINDS[act], float(limit), shared
+        self.gated, self.identity, self.groups, self.keep_groups = gated, int(identity), int(groups), int(keep_groups)
+        self.act_kind = GatedMLP.KINDS[act] if gated else ActMLP.KINDS[act]
+        self.limit, self.shared = float(limit), shared
 
     def load(self, stc, prefix: str, dtype, device, extra_parts=()):
         stack = lambda nm: torch.stack([_w(stc, f"{prefix}e{e}.{nm}", dtype, device) for e in range(self.experts)]).contiguous()
-        self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
+        self.w_gate, self.w_up, self.w_down = (stack("gate") if self.gated else None), stack("up"), stack("down")
         self.w_router = _f32(stc, prefix + "router", device)
         self.b_router = _f32(stc, prefix + "router.b", device) if self.has_router_bias else None
         self.correction = _f32(stc, prefix + "correction", device) if self.has_correction else None
         if self.shared is not None:
             self.shared.load(stc, prefix + "shared.", dtype, device)
         self.inp = FusedInput(list(extra_parts)) if extra_parts else None
-        assert self.w_gate.shape == (self.experts, self.ff, self.width) and self.w_down.shape == (self.experts, self.width, self.ff)
+        assert self.w_up.shape == (self.experts, self.ff, self.width) and self.w_down.shape == (self.experts, self.width, self.ff)
+        assert self.w_router.shape == (self.experts + self.identity, self.width)
         self.dtype = dtype
 
     def forward(self, h: torch.Tensor, sb: StepBatch) -> tuple[torch.Tensor, dict]:
@@ -426,12 +446,28 @@ class SparseExperts:
         logits = torch.addmm(self.b_router, hf, self.w_router.t()) if self.b_router is not None else torch.mm(hf, self.w_router.t())
         idx = torch.empty((sb.n, self.top), dtype=torch.int32, device=h.device)
         wts = torch.empty((sb.n, self.top), dtype=torch.float32, device=h.device)
+        idw = None                                                                  # per row: the weights of the chosen experts that return their input
         if self.router == "softmax":
             mix_ops.topk_softmax(idx, wts, logits)
-        else:
+        elif self.router == "sigmoid" and self.groups == 1 and not self.identity:
             mix_ops.topk_sigmoid(idx, wts, logits, self.correction, self.route_scale)
+        else:
+            idw = torch.empty((sb.n,), dtype=torch.float32, device=h.device) if self.identity else None
+            mix_ops.topk_grouped(idx, wts, idw, logits, self.correction, mix_ops.ROUTE_SOFTMAX_ALL if self.router == "softmax_all" else mix_ops.ROUTE_SIGMOID,
+                                 self.experts, self.groups, self.keep_groups, self.route_scale)
         y = torch.empty((sb.n, self.width), dtype=self.dtype, device=h.device)
-        if sb.n >= self.GROUPED_MIN_ROWS:
+        if not self.gated:
+            if sb.n >= self.GROUPED_MIN_ROWS:
+                mix_ops.moe_grouped_plain(y, h, self.w_up, self.w_down, idx, wts, self.act_kind, idw)
+            elif sb.n >= self.EXPERT_MAJOR_MIN_ROWS and mix_ops.moe_vector_layout(h, self.ff):
+                mix_ops.moe_expert_major_plain(y, h, self.w_up, self.w_down, idx, wts, self.act_kind, idw)
+            else:
+                hid = torch.empty((sb.n * self.top, self.ff), dtype=self.dtype, device=h.device)
+                mix_ops.moe_up_act(hid, h, self.w_up, idx, self.act_kind)
+                mix_ops.moe_down_id(y, hid, self.w_down, idx, wts, h, idw)
+        elif idw is not None:
+            raise RuntimeError("experts: the gated experts' kernels carry no identity share")
+        elif sb.n >= self.GROUPED_MIN_ROWS:
             mix_ops.moe_grouped(y, h, self.w_gate, self.w_up, self.w_down, idx, wts, self.act_kind, self.limit)
         elif sb.n >= self.EXPERT_MAJOR_MIN_ROWS and mix_ops.moe_vector_layout(h, self.ff):
             mix_ops.moe_expert_major(y, h, self.w_gate, self.w_up, self.w_down, idx, wts, self.act_kind, self.limit)
@@ -473,3 +509,127 @@ class GatedResidualBlock:
         h3 = torch.empty_like(h) if next_norm is not None else None
         mix_ops.gated_residual(x, y, p["rg"], next_norm, h3, self.eps)
         return h3
+
+
+class CanonNorm:
+    """What a sublayer reads in blocks with an input convolution: hn = x / sqrt(mean(x^2) + eps) * (1 + w), then h_t = hn_t + sum_j c[:, j] hn_(t - taps + 1 + j)
+    per channel, rows before the sequence's start being zero.  It is never a kernel chain of its own: the residual update before it writes it.  A step
+    of one row per sequence is ONE launch (update, norm, convolution against the slot's ring of the last taps - 1 normed rows, ring store); a prompt step is
+    two (update + norm of every row, then the convolution over the step's own rows)."""
+
+    def __init__(self, width: int, taps: int, eps: float):
+        if taps < 1 or taps > 16:
+            raise RuntimeError(f"input convolution: {taps} taps")
+        self.width, self.taps, self.eps = width, int(taps), float(eps)
+
+    def load(self, stc, norm_key: str, conv_key: str, dtype, device):
+        self.w = (1.0 + _f32(stc, norm_key, device)).contiguous()              # the stored weight lies around zero
+        self.conv = _f32(stc, conv_key, device)
+        assert self.w.numel() == self.width and self.conv.shape == (self.width, self.taps)
+        self.dtype = dtype
+        return self
+
+    def state_spec(self, name: str) -> StateSpec:
+        return StateSpec(name, (max(self.taps - 1, 1), self.width), self.dtype)
+
+    def apply(self, x: torch.Tensor, y: torch.Tensor | None, mode: int, sb: StepBatch, ring: torch.Tensor) -> torch.Tensor:
+        """x <- x | x + y | y, returns the sublayer's input [n, width] in the activation type."""
+        h = torch.empty((sb.n, self.width), dtype=self.dtype, device=x.device)
+        if sb.decode:
+            mix_ops.residual_rms(x, y, mode, self.w, self.eps, h, self.conv, ring, sb.tok_seq, sb.tok_pos, sb.slots)
+            return h
+        hn = torch.empty_like(h)
+        mix_ops.residual_rms(x, y, mode, self.w, self.eps, hn)
+        mix_ops.canon(h, hn, self.conv, ring, sb.tok_seq, sb.tok_pos, sb.slots, sb.pos0, sb.len_after)
+        return h
+
+
+class DifferentialAttention:
+    """H query heads over G key/value heads, every head with `maps` = 2 attention maps over the same values: q [H][2][dim], k [G][2][dim], v [G][vdim].
+    Queries and keys: bias, RMS norm per (head, map) with one weight for all, rotary positions on the first rot_dims entries (rotate-half pairs, optional
+    YaRN blend and magnitude).  score = scale q.k, soft-capped; mask = the row's own chunk of `span` positions ("chunk") or the last `span` positions
+    ("window"); plain softmax.  o = a1 - lambda a2 with lambda = exp(lq1.lk1) - exp(lq2.lk2) + diff, divided by its RMS over vdim, times (1 - diff), times
+    sigmoid(W_g h) per head; then W_o with bias.  Per slot: rings of `span` keys and values (entry = position mod span: with the chunk mask a row's chunk
+    is the entries 0 .. position mod span)."""
+    MAPS = 2
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, softcap: float, span: int, mask: str, diff: float, eps: float,
+                 rot_dims: int = 0, rot_base: float = 10000.0, rot_scaling: dict | None = None, gate: bool = True):
+        if heads % kv_heads:
+            raise RuntimeError(f"attention: {heads} query heads over {kv_heads} key/value heads")
+        if rot_dims % 2 or rot_dims > dim:
+            raise RuntimeError(f"attention: {rot_dims} rotated dimensions of {dim}")
+        if mask not in ("chunk", "window") or span < 1:
+            raise RuntimeError(f"attention: mask {mask!r} over {span} positions")
+        self.width, self.heads, self.kv_heads, self.dim, self.vdim = width, heads, kv_heads, dim, vdim
+        self.scale, self.softcap, self.span, self.diff, self.eps = float(scale), float(softcap or 0.0), int(span), float(diff), float(eps)
+        self.mask = mix_ops.MASK_CHUNK if mask == "chunk" else mix_ops.MASK_WINDOW
+        self.rot_dims, self.rot_base, self.rot_scaling, self.has_gate = int(rot_dims), float(rot_base), rot_scaling, gate
+
+    def load(self, stc, prefix: str, dtype, device, extra_parts=()):
+        parts = [(nm, _w(stc, prefix + nm, dtype, device), _w(stc, prefix + nm + ".b", dtype, device)) for nm in ("q", "k", "v")]
+        if self.has_gate:
+            parts.append(("g", _w(stc, prefix + "g", dtype, device), None))
+        self.inp = FusedInput(parts + list(extra_parts))
+        H, G, d, dv, M = self.heads, self.kv_heads, self.dim, self.vdim, self.MAPS
+        assert self.inp.offsets["q"][1] == H * M * d and self.inp.offsets["k"][1] == G * M * d and self.inp.offsets["v"][1] == G * dv
+        self.q_norm, self.k_norm = _f32(stc, prefix + "q.norm", device), _f32(stc, prefix + "k.norm", device)
+        l = {nm: stc.get_tensor(prefix + nm, device="cpu").to(torch.float64) for nm in ("lq1", "lk1", "lq2", "lk2")}
+        self.lam = float(torch.exp((l["lq1"] * l["lk1"]).sum()) - torch.exp((l["lq2"] * l["lk2"]).sum()) + self.diff)
+        self.w_o, self.b_o = _w(stc, prefix + "o", dtype, device), _w(stc, prefix + "o.b", dtype, device)
+        assert self.w_o.shape == (self.width, H * dv)
+        if self.rot_dims:
+            f, self.rot_mag = rotary_frequencies(self.rot_dims, self.rot_base, self.rot_scaling)
+            self.freq = f.to(device).contiguous()
+        else:
+            self.freq, self.rot_mag = None, 1.0
+        self.dtype = dtype
+
+    def state_specs(self) -> list[StateSpec]:
+        return [StateSpec("ring_k", (self.span, self.kv_heads * self.MAPS, self.dim), self.dtype), StateSpec("ring_v", (self.span, self.kv_heads, self.vdim), self.dtype)]
+
+    def forward(self, h: torch.Tensor, sb: StepBatch, state: dict) -> tuple[torch.Tensor, dict]:
+        H, G, d, dv, M = self.heads, self.kv_heads, self.dim, self.vdim, self.MAPS
+        p = self.inp(h)
+        mix_ops.qk_prep(p["q"], p["k"], p["v"], self.q_norm, self.k_norm, self.freq, self.rot_mag, False, self.eps, state["ring_k"], state["ring_v"],
+                        sb.tok_seq, sb.tok_pos, sb.slots, sb.len_after, d)
+        a = torch.empty((sb.n, H * M * dv), dtype=torch.float32, device=h.device)      # the maps' weighted sums stay float32 until they are combined
+        if sb.decode:
+            mix_ops.attn_decode_maps(a, p["q"], state["ring_k"], state["ring_v"], None, None, sb.slots, sb.len_after, H, M, self.scale, self.softcap, self.mask)
+        else:
+            mix_ops.attn_prefill_maps(a, p["q"], p["k"], p["v"], None, None, sb.cu, sb.tok_seq, sb.tok_pos, H, G, M, d, dv, self.scale, self.softcap, self.span,
+                                      self.mask, max_rows=sb.max_rows)
+        out = torch.empty((sb.n, H * dv), dtype=self.dtype, device=h.device)
+        mix_ops.diff_combine(out, a, self.lam, self.diff, self.eps, p.get("g"), H, dv)
+        return F.linear(out, self.w_o, self.b_o), p
+
+
+class CanonBlock:
+    """x += mixer(in1(x)); x += ff(in2(x)) (if a feed-forward), in1 / in2 being CanonNorm inputs.  The block is entered with its first input already
+    computed and leaves by computing the next block's (the residual update and the norm behind it are one kernel), or by the bare update."""
+
+    def __init__(self, width: int, eps: float, taps: int, mixer, mlp):
+        self.width, self.eps, self.mixer, self.mlp = width, float(eps), mixer, mlp
+        self.in1, self.in2 = CanonNorm(width, taps, eps), (CanonNorm(width, taps, eps) if mlp is not None else None)
+
+    def load(self, stc, prefix: str, dtype, device):
+        self.in1.load(stc, prefix + "norm1", prefix + "canon1", dtype, device)
+        self.mixer.load(stc, prefix + "mix.", dtype, device)
+        if self.mlp is not None:
+            self.in2.load(stc, prefix + "norm2", prefix + "canon2", dtype, device)
+            self.mlp.load(stc, prefix + "mlp.", dtype, device)
+        self.dtype = dtype
+
+    def state_specs(self) -> list[StateSpec]:
+        return self.mixer.state_specs() + [self.in1.state_spec("canon1")] + ([self.in2.state_spec("canon2")] if self.in2 is not None else [])
+
+    def forward(self, x: torch.Tensor, h: torch.Tensor, sb: StepBatch, state: dict, nxt: tuple | None) -> torch.Tensor | None:
+        """x: float32 residual (updated in place); h = in1(x).  nxt = (the next block's in1, its ring): returns the next block's input; None: returns None."""
+        y, _ = self.mixer.forward(h, sb, state)
+        if self.mlp is not None:
+            h2 = self.in2.apply(x, y, mix_ops.RES_ADD, sb, state["canon2"])
+            y, _ = self.mlp.forward(h2, sb)
+        if nxt is None:
+            mix_ops.residual_rms(x, y, mix_ops.RES_ADD, None, self.eps, None)
+            return None
+        return nxt[0].apply(x, y, mix_ops.RES_ADD, sb, nxt[1])

@@ -42,7 +42,12 @@ extern "C" {
 #define EXL3_MIX_ACT_GELU_TANH 1
 #define EXL3_MIX_ACT_SILU      2
 
-#define EXL3_MIX_ABI_VERSION 2
+/* attention masks: WINDOW: a row sees the last `window` positions up to itself; CHUNK: the positions up to itself inside its own chunk of `window`
+ * positions, chunks counted from position 0 of the sequence. */
+#define EXL3_MIX_MASK_WINDOW 0
+#define EXL3_MIX_MASK_CHUNK  1
+
+#define EXL3_MIX_ABI_VERSION 3
 
 const char* exl3_mix_last_error(void);
 int  exl3_mix_abi_version(void);
@@ -196,6 +201,72 @@ int exl3_mix_latent_decode_mfma_scratch(int n, int heads, int rank, int splits, 
 int exl3_mix_latent_decode_mfma(void* o_lat, int64_t o_row, int64_t o_head, const void* q_lat, int64_t ql_row, int64_t ql_head, const void* q, int64_t q_ld,
                                 const void* ring, const float* sink, const int32_t* slots, const int32_t* len_after, float* scratch, int splits,
                                 int n, int heads, int dim, int rot_dim, int rank, float scale, int window, void* stream);
+
+/* ---- several attention maps per head, chunk masks, soft-capped scores (mix_attn.hip, mix_attn_mfma.hip, mix_diffattn.hip) ---- */
+
+/* The attention kernels above with: `maps` maps per head (queries [n][heads][maps][dim], keys [.][kv_heads][maps][dim]; every map of a head reads the values
+ * of the head's key/value head; out [n][heads][maps][vdim]; a gate needs maps == 1), scores soft-capped to softcap tanh(score / softcap) (softcap 0: none),
+ * mask EXL3_MIX_MASK_* over `window` positions, values as a column block (v_ld), and the result in float32 (out_f32) or the activation type.
+ * Decode with the chunk mask reads the ring entries 0 .. (len_after - 1) % window. */
+int exl3_mix_attn_prefill_ex(void* out, int out_f32, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v, int64_t v_ld,
+                             const void* gate, int64_t gate_ld, const float* sink, const int32_t* cu, const int32_t* tok_seq, const int32_t* tok_pos,
+                             int n, int heads, int kv_heads, int maps, int dim, int vdim, float scale, float softcap, int window, int mask, int dtype, void* stream);
+int exl3_mix_attn_prefill_mfma_ex(void* out, int out_f32, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v, int64_t v_ld,
+                                  const void* gate, int64_t gate_ld, const float* sink, const int32_t* cu,
+                                  int batch, int max_rows, int heads, int kv_heads, int maps, int dim, int vdim, float scale, float softcap, int window, int mask,
+                                  void* stream);
+int exl3_mix_attn_decode_ex(void* out, int out_f32, const void* q, int64_t q_ld, const void* ring_k, const void* ring_v,
+                            const void* gate, int64_t gate_ld, const float* sink, const int32_t* slots, const int32_t* len_after,
+                            int n, int heads, int kv_heads, int maps, int dim, int vdim, float scale, float softcap, int window, int mask, int dtype, void* stream);
+
+/* Queries and keys before the attention core, in place: per (row, head) RMS norm over dim with the weight q_norm / k_norm [dim] (NULL: none), then rotary
+ * positions on the first rot_dims entries (freq [rot_dims / 2], NULL: none): pairs (i, i + rot_dims/2), or (2i, 2i+1) when `interleaved`; angle =
+ * tok_pos * freq[i], cos and sin times `mag`.  q_heads and k_heads count every (head, map).  Keys and values of the rows with tok_pos >= len_after - window
+ * go to ring_k [slots][window][k_heads][dim] and ring_v [slots][window][v_heads][vdim] at tok_pos % window. */
+int exl3_mix_qk_prep(void* q, int64_t q_ld, void* k, int64_t k_ld, const void* v, int64_t v_ld, const float* q_norm, const float* k_norm,
+                     const float* freq, int rot_dims, float mag, int interleaved, float eps, void* ring_k, void* ring_v,
+                     const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots, const int32_t* len_after,
+                     int n, int q_heads, int k_heads, int v_heads, int dim, int vdim, int window, int dtype, void* stream);
+
+/* Differential attention: a [n][heads][2][vdim] float32 (the two maps of every head);  o = a1 - lambda a2;
+ * out[n][h][c] = o_c / sqrt(mean_c(o^2) + eps) * (1 - diff) * sigmoid(gate[n][h])  (gate NULL: no gate). */
+int exl3_mix_diff_combine(void* out, const float* a, float lambda, float diff, float eps, const void* gate, int64_t gate_ld,
+                          int n, int heads, int vdim, int dtype, void* stream);
+
+/* ---- pre-norm blocks with a short causal input convolution (mix_canon.hip) ---- */
+
+/* Residual update fused with the next RMS norm: mode 0: x stays; 1: x += y; 2: x = y.  If h: hn = x / sqrt(mean(x^2) + eps) * w.  Without conv_w, h = hn.
+ * With conv_w [width][taps] (steps of ONE row per sequence): h = hn + sum_j conv_w[c][j] hn_(pos - taps + 1 + j), the earlier rows read from
+ * ring [slots][taps - 1][width] (entry = position % (taps - 1); positions below 0 are zero rows), and hn is stored there. */
+int exl3_mix_residual_rms(float* x, const void* y, int64_t y_ld, int mode, const float* w, float eps, void* h, int64_t h_ld,
+                          const float* conv_w, int taps, void* ring, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots,
+                          int n, int width, int dtype, void* stream);
+
+/* The same convolution over a packed step whose sequences start in it (or bring one row each): out = hn + conv(hn), predecessors from the step's own rows
+ * where tok_pos - back >= pos0[seq], from the ring otherwise; the rows at the last taps - 1 positions of every sequence are stored in the ring. */
+int exl3_mix_canon(void* out, int64_t out_ld, const void* hn, int64_t hn_ld, const float* conv_w, int taps, void* ring,
+                   const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots, const int32_t* pos0, const int32_t* len_after,
+                   int n, int width, int dtype, void* stream);
+
+/* ---- routers over groups of experts, experts without weights, ungated experts (mix_rowops.hip, mix_moe.hip) ---- */
+
+/* Router over `total` outputs: the first `real` name stored experts, the others experts that return their input.  Scores s: softmax over all outputs
+ * (kind 0) or sigmoids (kind 1); the choice looks at s + correction (NULL: s); the outputs form `groups` equal groups of neighbours, a group counts as
+ * its largest choice score and only the `keep` best groups can be chosen from; the `top` best are taken (ties to the lower index); weights = chosen s /
+ * (their sum + 1e-20) * scale (normalise 0: s * scale).  A choice >= real is written as idx = real with weight 0, and idw[n] = the sum of such weights. */
+int exl3_mix_topk_grouped(int32_t* idx, float* wts, float* idw, const float* logits, const float* correction, int kind, float scale, int normalise,
+                          int groups, int keep, int n, int total, int real, int top, void* stream);
+
+/* Ungated experts: hid[n*top + r] = act(Wu[e] h[n]) (EXL3_MIX_ACT_*).  In all experts' kernels a choice outside 0 .. experts-1 is skipped. */
+int exl3_mix_moe_up_act(void* hid, const void* h, const void* wu, const int32_t* idx, int n, int top, int experts, int ff, int width, int act, int dtype, void* stream);
+int exl3_mix_moe_expert_major_plain(void* per, void* hid, const void* h, const void* wu, const void* wd, const int32_t* idx,
+                                    int n, int top, int experts, int ff, int width, int act, int dtype, void* stream);
+/* exl3_mix_moe_down / exl3_mix_moe_combine with y[n] += idw[n] * h_id[n] (idw NULL: nothing added); combine skips the choices that idx (NULL: none)
+ * places outside 0 .. experts-1. */
+int exl3_mix_moe_down_id(void* y, const void* hid, const void* wd, const int32_t* idx, const float* wts, const void* h_id, const float* idw,
+                         int n, int top, int experts, int ff, int width, int dtype, void* stream);
+int exl3_mix_moe_combine_id(void* y, const void* sorted, const int32_t* where, const float* wts, const int32_t* idx, int experts, const void* h_id,
+                            const float* idw, int n, int top, int width, int dtype, void* stream);
 
 #ifdef __cplusplus
 }
