@@ -521,6 +521,7 @@ class CanonNorm:
         if taps < 1 or taps > 16:
             raise RuntimeError(f"input convolution: {taps} taps")
         self.width, self.taps, self.eps = width, int(taps), float(eps)
+        self.dtype = torch.bfloat16                                  # until load() says otherwise
 
     def load(self, stc, norm_key: str, conv_key: str, dtype, device):
         self.w = (1.0 + _f32(stc, norm_key, device)).contiguous()              # the stored weight lies around zero
@@ -565,6 +566,7 @@ class DifferentialAttention:
         self.scale, self.softcap, self.span, self.diff, self.eps = float(scale), float(softcap or 0.0), int(span), float(diff), float(eps)
         self.mask = mix_ops.MASK_CHUNK if mask == "chunk" else mix_ops.MASK_WINDOW
         self.rot_dims, self.rot_base, self.rot_scaling, self.has_gate = int(rot_dims), float(rot_base), rot_scaling, gate
+        self.dtype = torch.bfloat16                                  # until load() says otherwise
 
     def load(self, stc, prefix: str, dtype, device, extra_parts=()):
         parts = [(nm, _w(stc, prefix + nm, dtype, device), _w(stc, prefix + nm + ".b", dtype, device)) for nm in ("q", "k", "v")]
