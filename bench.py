@@ -57,7 +57,9 @@ def parse():
                     help="instead of the default workload: layer times of the unquantized mixer family (Vofanex) beside the EXL3 Llama layer of equal size, and its kernels' rooflines")
     ap.add_argument("--latent-family", action="store_true",
                     help="instead of the default workload: layer times of the latent-attention family (Zagilorn) beside Vofanex layers of equal size, and its kernels' rooflines")
-    ap.add_argument("--mixer-sizes", default="", help="with --mixer-family: comma-separated sizes (1b, 8b; default both)")
+    ap.add_argument("--diff-family", action="store_true",
+                    help="instead of the default workload: layer times of the differential-attention family (Fimunex) beside Vofanex layers of equal size, and its kernels' rooflines")
+    ap.add_argument("--mixer-sizes", default="", help="with --mixer-family / --latent-family / --diff-family: comma-separated sizes (1b, 8b; default both)")
     ap.add_argument("--variant", type=int, default=1)
     ap.add_argument("--attention", action="store_true", help="include decode attention over the quantized KV cache (context = 1000 tokens) in the timed step")
     ap.add_argument("--unfused", action="store_true", help="one launch per reference op instead of the fused pipeline")
@@ -259,6 +261,9 @@ def main():
     if args.latent_family:
         from exllamav3_amd import latent_bench
         sys.exit(latent_bench.run(args))
+    if args.diff_family:
+        from exllamav3_amd import diff_bench
+        sys.exit(diff_bench.run(args))
     import torch
     from exllamav3_amd import ext
     from exllamav3_amd.llama_path import SHAPES, SyntheticEXL3Llama

@@ -338,3 +338,4 @@ def _declare_mix(l):
     sig("exl3_mix_moe_expert_major_plain", vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp)
     sig("exl3_mix_moe_down_id", vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp)
     sig("exl3_mix_moe_combine_id", vp, vp, vp, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp)
+    sig("exl3_mix_softcap", vp, i64, f32, vp)

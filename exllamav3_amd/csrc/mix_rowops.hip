@@ -274,6 +274,12 @@ __global__ __launch_bounds__(64) void topk_grouped_kernel(int32_t* __restrict__ 
     if (idw && lane == 0) idw[n] = iw;
 }
 
+// x <- cap * tanh(x / cap) over float32 values (logits), in place
+__global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, int64_t count, float cap)
+{
+    for (int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t) gridDim.x * 256) x[i] = cap * tanhf(x[i] / cap);
+}
+
 extern "C" int exl3_mix_embed_copy(float* x, void* xc, int64_t xc_ld, const void* table, const int32_t* tokens, int n, int width, int vocab, int dtype, void* stream)
 {
     MIX_CHECK(x && table && tokens && n >= 0 && width > 0 && vocab > 0 && (!xc || xc_ld >= width), "mix_embed_copy: bad arguments");
@@ -376,4 +382,13 @@ extern "C" int exl3_mix_topk_grouped(int32_t* idx, float* wts, float* idw, const
     if (n == 0) return EXL3_MIX_OK;
     hipLaunchKernelGGL(topk_grouped_kernel, dim3(n), dim3(64), 0, (hipStream_t) stream, idx, wts, idw, logits, correction, kind, scale, normalise, groups, keep, total, real, top);
     return mix_check_launch("mix_topk_grouped");
+}
+
+extern "C" int exl3_mix_softcap(float* x, int64_t count, float cap, void* stream)
+{
+    MIX_CHECK(x && count >= 0 && cap > 0.f, "mix_softcap: bad arguments");
+    if (count == 0) return EXL3_MIX_OK;
+    const int blocks = (int) ((count + 255) / 256 > 4096 ? 4096 : (count + 255) / 256);
+    hipLaunchKernelGGL(softcap_kernel, dim3(blocks), dim3(256), 0, (hipStream_t) stream, x, count, cap);
+    return mix_check_launch("mix_softcap");
 }

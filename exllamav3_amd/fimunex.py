@@ -131,5 +131,5 @@ class FimunexModel:
         mix_ops.rms_norm_rows(hw, x, sb.want_rows, self.final_norm, self.cfg.eps)
         logits = F.linear(hw, self.head).float()
         if self.cfg.logit_softcap:
-            logits = self.cfg.logit_softcap * torch.tanh(logits / self.cfg.logit_softcap)
+            mix_ops.softcap(logits, self.cfg.logit_softcap)
         return logits

@@ -525,6 +525,12 @@ def canon(out, hn, conv_w, ring, tok_seq, tok_pos, slots, pos0, len_after):
                                          _p(pos0), _p(len_after), n, width, code(hn.dtype), _stream(hn)))
 
 
+def softcap(x: torch.Tensor, cap: float):
+    """x <- cap tanh(x / cap) in place (float32, contiguous)."""
+    _f32c(x, "x")
+    _check(_lib.mixlib().exl3_mix_softcap(_p(x), x.numel(), cap, _stream(x)))
+
+
 # ---- grouped routers, experts without weights, ungated experts (csrc/mix_rowops.hip, mix_moe.hip) ------------------------------------------------------
 ROUTE_SOFTMAX_ALL, ROUTE_SIGMOID = 0, 1
 

@@ -248,6 +248,9 @@ int exl3_mix_canon(void* out, int64_t out_ld, const void* hn, int64_t hn_ld, con
                    const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots, const int32_t* pos0, const int32_t* len_after,
                    int n, int width, int dtype, void* stream);
 
+/* x <- cap * tanh(x / cap) over `count` float32 values in place (soft-capped logits). */
+int exl3_mix_softcap(float* x, int64_t count, float cap, void* stream);
+
 /* ---- routers over groups of experts, experts without weights, ungated experts (mix_rowops.hip, mix_moe.hip) ---- */
 
 /* Router over `total` outputs: the first `real` name stored experts, the others experts that return their input.  Scores s: softmax over all outputs
