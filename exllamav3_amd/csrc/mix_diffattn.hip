@@ -1,5 +1,5 @@
 // Around the attention core of heads that carry normed, rotated queries and keys and several attention maps per head:
-//   qk_prep        per (row, head, map): RMS norm of the query / key over its dim with a weight shared by all heads, rotary positions on the first
+//   qk_prep        per row, for every (head, map): RMS norm of the query / key over its dim with a weight shared by all heads, rotary positions on the first
 //                  rot_dims entries (pairs (i, i + rot_dims/2), or interleaved pairs), in place; keys and values of the rows a sequence keeps go into
 //                  the slot's rings.
 //   diff_combine   differential attention: o = a1 - lambda a2 of a head's two maps, divided by its root mean square over the value dim, times
@@ -7,63 +7,73 @@
 // Sums of squares, angles, cos / sin and the combination are float32.
 #include "mix_common.cuh"
 
-// grid (rows, q_heads + k_heads + v_heads), one wave.  q [n][q_heads][dim], k [n][k_heads][dim], v [n][v_heads][vdim] are column blocks of wider
-// matrices (row strides); q_heads and k_heads count (head, map).  ring_k [slots][window][k_heads][dim], ring_v [slots][window][v_heads][vdim],
+// One workgroup of QP_WAVES waves per row: cos / sin of the row's position are computed once into LDS, then the waves take the row's items -- q_heads
+// query vectors, k_heads key vectors, v_heads value vectors -- in turn.  q [n][q_heads][dim], k [n][k_heads][dim], v [n][v_heads][vdim] are column blocks
+// of wider matrices (row strides); q_heads and k_heads count (head, map).  ring_k [slots][window][k_heads][dim], ring_v [slots][window][v_heads][vdim],
 // entry = position % window, written for the rows with position >= len_after - window.
+#define QP_WAVES 4
 template <typename T>
-__global__ __launch_bounds__(64) void qk_prep_kernel(T* __restrict__ q, int64_t q_ld, T* __restrict__ k, int64_t k_ld, const T* __restrict__ v, int64_t v_ld,
+__global__ __launch_bounds__(64 * QP_WAVES) void qk_prep_kernel(T* __restrict__ q, int64_t q_ld, T* __restrict__ k, int64_t k_ld, const T* __restrict__ v, int64_t v_ld,
                                                      const float* __restrict__ q_norm, const float* __restrict__ k_norm, const float* __restrict__ freq, int rot_dims,
                                                      float mag, int interleaved, float eps, T* __restrict__ ring_k, T* __restrict__ ring_v,
                                                      const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ slots,
                                                      const int32_t* __restrict__ len_after, int q_heads, int k_heads, int v_heads, int dim, int vdim, int window)
 {
-    extern __shared__ float buf[];                            // [dim]
-    const int n = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
+    extern __shared__ float smem[];                           // cos [rot_dims / 2] | sin [rot_dims / 2] | per wave: a vector [dim]
+    const int n = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int half = freq ? rot_dims >> 1 : 0;
+    float* cs = smem;
+    float* sn = smem + half;
+    float* buf = smem + 2 * half + wv * dim;
     const int b = tok_seq[n], pos = tok_pos[n];
     const bool keep = pos >= len_after[b] - window;
     const int64_t ring_row = (int64_t) slots[b] * window + (pos % window);
-    if (item >= q_heads + k_heads)
+    for (int p = threadIdx.x; p < half; p += 64 * QP_WAVES)
     {
-        if (!keep) return;
-        const int g = item - q_heads - k_heads;
-        const T* vr = v + (int64_t) n * v_ld + (int64_t) g * vdim;
-        T* rv = ring_v + (ring_row * v_heads + g) * vdim;
-        for (int i = lane; i < vdim; i += 64) rv[i] = vr[i];
-        return;
-    }
-    const bool is_q = item < q_heads;
-    const int head = is_q ? item : item - q_heads;
-    T* vec = is_q ? q + (int64_t) n * q_ld + (int64_t) head * dim : k + (int64_t) n * k_ld + (int64_t) head * dim;
-    const float* nw = is_q ? q_norm : k_norm;
-    float ss = 0.f;
-    for (int i = lane; i < dim; i += 64) { const float x = to_f(vec[i]); buf[i] = x; ss += x * x; }
-    if (nw)
-    {
-        ss = wave_sum(ss);
-        const float inv = 1.0f / sqrtf(ss / (float) dim + eps);
-        for (int i = lane; i < dim; i += 64) buf[i] = buf[i] * inv * nw[i];
+        const float a = (float) pos * freq[p];
+        cs[p] = cosf(a) * mag; sn[p] = sinf(a) * mag;
     }
     __syncthreads();
-    if (freq)
+    const int items = q_heads + k_heads + (keep ? v_heads : 0);
+    for (int item = wv; item < items; item += QP_WAVES)
     {
-        const int half = rot_dims >> 1;
+        if (item >= q_heads + k_heads)
+        {
+            const int g = item - q_heads - k_heads;
+            const T* vr = v + (int64_t) n * v_ld + (int64_t) g * vdim;
+            T* rv = ring_v + (ring_row * v_heads + g) * vdim;
+            for (int i = lane; i < vdim; i += 64) rv[i] = vr[i];
+            continue;
+        }
+        const bool is_q = item < q_heads;
+        const int head = is_q ? item : item - q_heads;
+        T* vec = is_q ? q + (int64_t) n * q_ld + (int64_t) head * dim : k + (int64_t) n * k_ld + (int64_t) head * dim;
+        const float* nw = is_q ? q_norm : k_norm;
+        float ss = 0.f;
+        for (int i = lane; i < dim; i += 64) { const float x = to_f(vec[i]); buf[i] = x; ss += x * x; }
+        if (nw)
+        {
+            ss = wave_sum(ss);
+            const float inv = 1.0f / sqrtf(ss / (float) dim + eps);
+            for (int i = lane; i < dim; i += 64) buf[i] = buf[i] * inv * nw[i];
+        }
+        __builtin_amdgcn_wave_barrier();                      // LDS serves a wave's accesses in order: the stores above are visible to the reads below
         for (int p = lane; p < half; p += 64)
         {
-            const float a = (float) pos * freq[p];
-            const float c = cosf(a) * mag, s = sinf(a) * mag;
             const int i0 = interleaved ? 2 * p : p, i1 = interleaved ? 2 * p + 1 : p + half;
-            const float u = buf[i0], w = buf[i1];
+            const float u = buf[i0], w = buf[i1], c = cs[p], s = sn[p];
             buf[i0] = u * c - w * s;
             buf[i1] = w * c + u * s;
         }
-        __syncthreads();
-    }
-    T* rk = (!is_q && keep) ? ring_k + (ring_row * k_heads + head) * dim : nullptr;
-    for (int i = lane; i < dim; i += 64)
-    {
-        const T o = from_f<T>(buf[i]);
-        vec[i] = o;
-        if (rk) rk[i] = o;
+        __builtin_amdgcn_wave_barrier();
+        T* rk = (!is_q && keep) ? ring_k + (ring_row * k_heads + head) * dim : nullptr;
+        for (int i = lane; i < dim; i += 64)
+        {
+            const T o = from_f<T>(buf[i]);
+            vec[i] = o;
+            if (rk) rk[i] = o;
+        }
+        __builtin_amdgcn_wave_barrier();                      // the next item overwrites buf
     }
 }
 
@@ -90,12 +100,13 @@ extern "C" int exl3_mix_qk_prep(void* q, int64_t q_ld, void* k, int64_t k_ld, co
                                 int n, int q_heads, int k_heads, int v_heads, int dim, int vdim, int window, int dtype, void* stream)
 {
     MIX_CHECK(q && k && v && ring_k && ring_v && tok_seq && tok_pos && slots && len_after, "mix_qk_prep: null pointer");
-    MIX_CHECK(n >= 0 && q_heads > 0 && k_heads > 0 && v_heads > 0 && q_heads + k_heads + v_heads <= 65535 && dim > 0 && dim <= 8192 && vdim > 0 && window > 0,
+    MIX_CHECK(n >= 0 && q_heads > 0 && k_heads > 0 && v_heads > 0 && dim > 0 && dim <= 2048 && vdim > 0 && window > 0,
               "mix_qk_prep: bad sizes");
     MIX_CHECK(q_ld >= (int64_t) q_heads * dim && k_ld >= (int64_t) k_heads * dim && v_ld >= (int64_t) v_heads * vdim, "mix_qk_prep: bad row strides");
     MIX_CHECK(!freq || (rot_dims >= 2 && rot_dims % 2 == 0 && rot_dims <= dim), "mix_qk_prep: %d rotated entries of %d", rot_dims, dim);
     if (n == 0) return EXL3_MIX_OK;
-    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(qk_prep_kernel<T>, dim3(n, q_heads + k_heads + v_heads), dim3(64), (size_t) dim * sizeof(float), (hipStream_t) stream,
+    const size_t sm = (size_t) ((freq ? rot_dims : 0) + QP_WAVES * dim) * sizeof(float);
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(qk_prep_kernel<T>, dim3(n), dim3(64 * QP_WAVES), sm, (hipStream_t) stream,
                                              (T*) q, q_ld, (T*) k, k_ld, (const T*) v, v_ld, q_norm, k_norm, freq, rot_dims, mag, interleaved, eps, (T*) ring_k, (T*) ring_v,
                                              tok_seq, tok_pos, slots, len_after, q_heads, k_heads, v_heads, dim, vdim, window));
     return mix_check_launch("mix_qk_prep");

@@ -110,7 +110,7 @@ def diff_kernel_legs(size_name: str, prompt: int, ctx: int, dev):
         od, gd = torch.empty((bs, H * dv), dtype=bf, device=dev), rnd(bs, H)
         t = _time(lambda: mix_ops.diff_combine(od, ad, 0.7, 0.6, 1e-5, gd, H, dv), 50)
         out[f"diff_combine_bs{bs}"] = {"us": t * 1e6}
-    x, y, nw, cw = torch.randn(n, w, device=dev), rnd(n, w), torch.ones(w, device=dev), 0.3 * torch.randn(w, TAPS, device=dev)
+    x, y, nw, cw = torch.randn(n, w, device=dev), rnd(n, w), torch.ones(w, device=dev), 0.3 * torch.randn(TAPS, w, device=dev)
     hn, h, ring = torch.empty((n, w), dtype=bf, device=dev), torch.empty((n, w), dtype=bf, device=dev), torch.zeros((16, TAPS - 1, w), dtype=bf, device=dev)
     t1 = _time(lambda: mix_ops.residual_rms(x, y, mix_ops.RES_ADD, nw, 1e-5, hn), 20)
     t2 = _time(lambda: mix_ops.canon(h, hn, cw, ring, seq, pos, sl, p0, la), 20)

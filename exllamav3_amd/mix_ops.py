@@ -490,8 +490,8 @@ def diff_combine(out, a, lam: float, diff: float, eps: float, gate_view, heads: 
 
 # ---- residual update + RMS norm + short causal input convolution (csrc/mix_canon.hip) ----------------------------------------------------------------
 def residual_rms(x, y_view, mode: int, w, eps: float, h_view, conv_w=None, ring=None, tok_seq=None, tok_pos=None, slots=None):
-    """x (float32, in place) = x | x + y | y (RES_*); h = rms_norm(x) * w, and with conv_w (steps of one row per sequence) h + its causal convolution over
-    the ring [slots, taps - 1, width] of earlier normed rows, which also receives the new one.  h_view None: the update alone."""
+    """x (float32, in place) = x | x + y | y (RES_*); h = rms_norm(x) * w, and with conv_w [taps, width] (steps of one row per sequence) h + its causal
+    convolution over the ring [slots, taps - 1, width] of earlier normed rows, which also receives the new one.  h_view None: the update alone."""
     n, width = x.shape
     _f32c(x, "x")
     ref = y_view if y_view is not None else h_view
@@ -502,8 +502,8 @@ def residual_rms(x, y_view, mode: int, w, eps: float, h_view, conv_w=None, ring=
         _f32c(w, "w"); _req(w.numel() == width and h_view.shape[0] == n and h_view.dtype == ref.dtype, "residual_rms: h / w")
     taps = 0
     if conv_w is not None:
-        _f32c(conv_w, "conv_w"); taps = conv_w.shape[1]
-        _req(conv_w.shape[0] == width and ring is not None and ring.is_contiguous() and ring.shape[1:] == (max(taps - 1, 1), width) and ring.dtype == ref.dtype,
+        _f32c(conv_w, "conv_w"); taps = conv_w.shape[0]
+        _req(conv_w.shape[1] == width and ring is not None and ring.is_contiguous() and ring.shape[1:] == (max(taps - 1, 1), width) and ring.dtype == ref.dtype,
              "residual_rms: convolution weights / ring")
         for t, nm in ((tok_seq, "tok_seq"), (tok_pos, "tok_pos"), (slots, "slots")):
             _i32c(t, nm)
@@ -513,11 +513,12 @@ def residual_rms(x, y_view, mode: int, w, eps: float, h_view, conv_w=None, ring=
 
 
 def canon(out, hn, conv_w, ring, tok_seq, tok_pos, slots, pos0, len_after):
-    """out = hn + causal convolution of hn over time per channel (conv_w [width, taps]) for a packed step; the ring keeps each sequence's last taps - 1 rows."""
+    """out = hn + causal convolution of hn over time per channel (conv_w [taps, width]: tap-major) for a packed step; the ring keeps each sequence's last
+    taps - 1 rows."""
     n, width = hn.shape
-    taps = conv_w.shape[1]
+    taps = conv_w.shape[0]
     _f32c(conv_w, "conv_w")
-    _req(out.shape == hn.shape and out.dtype == hn.dtype == ring.dtype and conv_w.shape[0] == width and ring.is_contiguous() and ring.shape[1:] == (max(taps - 1, 1), width),
+    _req(out.shape == hn.shape and out.dtype == hn.dtype == ring.dtype and conv_w.shape[1] == width and ring.is_contiguous() and ring.shape[1:] == (max(taps - 1, 1), width),
          "canon: shapes")
     for t, nm in ((tok_seq, "tok_seq"), (tok_pos, "tok_pos"), (slots, "slots"), (pos0, "pos0"), (len_after, "len_after")):
         _i32c(t, nm)

@@ -236,13 +236,13 @@ int exl3_mix_diff_combine(void* out, const float* a, float lambda, float diff, f
 /* ---- pre-norm blocks with a short causal input convolution (mix_canon.hip) ---- */
 
 /* Residual update fused with the next RMS norm: mode 0: x stays; 1: x += y; 2: x = y.  If h: hn = x / sqrt(mean(x^2) + eps) * w.  Without conv_w, h = hn.
- * With conv_w [width][taps] (steps of ONE row per sequence): h = hn + sum_j conv_w[c][j] hn_(pos - taps + 1 + j), the earlier rows read from
+ * With conv_w [taps][width] (steps of ONE row per sequence): h = hn + sum_j conv_w[j][c] hn_(pos - taps + 1 + j), the earlier rows read from
  * ring [slots][taps - 1][width] (entry = position % (taps - 1); positions below 0 are zero rows), and hn is stored there. */
 int exl3_mix_residual_rms(float* x, const void* y, int64_t y_ld, int mode, const float* w, float eps, void* h, int64_t h_ld,
                           const float* conv_w, int taps, void* ring, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots,
                           int n, int width, int dtype, void* stream);
 
-/* The same convolution over a packed step whose sequences start in it (or bring one row each): out = hn + conv(hn), predecessors from the step's own rows
+/* The same convolution (conv_w [taps][width]) over a packed step whose sequences start in it (or bring one row each): out = hn + conv(hn), predecessors from the step's own rows
  * where tok_pos - back >= pos0[seq], from the ring otherwise; the rows at the last taps - 1 positions of every sequence are stored in the ring. */
 int exl3_mix_canon(void* out, int64_t out_ld, const void* hn, int64_t hn_ld, const float* conv_w, int taps, void* ring,
                    const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots, const int32_t* pos0, const int32_t* len_after,
