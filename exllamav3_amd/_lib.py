@@ -339,3 +339,4 @@ def _declare_mix(l):
     sig("exl3_mix_moe_down_id", vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp)
     sig("exl3_mix_moe_combine_id", vp, vp, vp, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp)
     sig("exl3_mix_softcap", vp, i64, f32, vp)
+    sig("exl3_mix_attn_prefill_mfma_diff", vp, vp, i64, vp, i64, vp, i64, vp, i64, vp, i32, i32, i32, i32, i32, i32, f32, f32, i32, i32, f32, f32, f32, vp)

@@ -96,6 +96,9 @@ def diff_kernel_legs(size_name: str, prompt: int, ctx: int, dev):
         t = _time(lambda: mix_ops.attn_prefill_maps(a, q, k, v, None, None, cu, seq, pos, H, G, 2, d, dv, d ** -0.5, cap, C, mix_ops.MASK_CHUNK, max_rows=n, mfma=True), 10)
         out["attn_prefill_mfma_two_maps_chunk" + ("_softcap" if cap else "_no_softcap")] = {"ms": t * 1e3, "tflops": fl / t / 1e12, "of_bf16_peak": fl / t / PEAK_BF16}
     o, gt = torch.empty((n, H * dv), dtype=bf, device=dev), rnd(n, H)
+    for cap in (50.0, 0.0):
+        t = _time(lambda: mix_ops.attn_prefill_diff(o, q, k, v, gt, cu, H, G, d, dv, d ** -0.5, cap, C, mix_ops.MASK_CHUNK, 0.7, 0.6, 1e-5, n), 10)
+        out["attn_prefill_mfma_diff_fused" + ("_softcap" if cap else "_no_softcap")] = {"ms": t * 1e3, "tflops": fl / t / 1e12, "of_bf16_peak": fl / t / PEAK_BF16}
     t = _time(lambda: mix_ops.diff_combine(o, a, 0.7, 0.6, 1e-5, gt, H, dv), 20)
     out["diff_combine_prefill"] = hbm(n * H * dv * (2 * 4 + 2), t)
     for bs in (1, 16):

@@ -461,6 +461,24 @@ def attn_prefill_maps(out, q_view, k_view, v_view, gate_view, sink, cu, tok_seq,
                                                    n, heads, kv_heads, maps, dim, vdim, scale, softcap, window, mask, code(q_view.dtype), _stream(out)))
 
 
+def diff_mfma_ok(dtype, max_rows: int, dim: int, vdim: int, scale: float) -> bool:
+    return dtype == torch.bfloat16 and max_rows >= ATTN_MFMA_MIN_ROWS and dim <= 128 and vdim <= 256 and scale > 0
+
+
+def attn_prefill_diff(out, q_view, k_view, v_view, gate_view, cu, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, softcap: float, window: int, mask: int,
+                      lam: float, diff: float, eps: float, max_rows: int):
+    """Prompt-step differential attention on the matrix cores (bfloat16): both maps of every head and their combination in one kernel; out [n, heads * vdim]."""
+    n = q_view.shape[0]
+    _req(out.is_contiguous() and out.shape == (n, heads * vdim) and out.dtype == q_view.dtype == k_view.dtype == v_view.dtype == torch.bfloat16 and max_rows > 0,
+         "attn_prefill_diff: bfloat16 tensors and the step's longest sequence")
+    _req(k_view.shape[0] == n and v_view.shape[0] == n, "attn_prefill_diff: step tensors")
+    if gate_view is not None:
+        _req(gate_view.dtype == out.dtype and gate_view.shape[0] == n, "attn_prefill_diff: gate")
+    _check(_lib.mixlib().exl3_mix_attn_prefill_mfma_diff(_p(out), _p(q_view), _view(q_view, heads * 2 * dim, "q"), _p(k_view), _view(k_view, kv_heads * 2 * dim, "k"), _p(v_view),
+                                                          _view(v_view, kv_heads * vdim, "v"), _p(gate_view), 0 if gate_view is None else _view(gate_view, heads, "gate"), _p(cu),
+                                                          cu.numel() - 1, max_rows, heads, kv_heads, dim, vdim, scale, softcap, window, mask, lam, diff, eps, _stream(out)))
+
+
 def attn_decode_maps(out, q_view, ring_k, ring_v, gate_view, sink, slots, len_after, heads: int, maps: int, scale: float, softcap: float, mask: int):
     """One new row per sequence against the rings (ring_k [slots, window, kv_heads * maps, dim], ring_v [slots, window, kv_heads, vdim])."""
     n = out.shape[0]

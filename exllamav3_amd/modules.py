@@ -595,13 +595,18 @@ class DifferentialAttention:
         p = self.inp(h)
         mix_ops.qk_prep(p["q"], p["k"], p["v"], self.q_norm, self.k_norm, self.freq, self.rot_mag, False, self.eps, state["ring_k"], state["ring_v"],
                         sb.tok_seq, sb.tok_pos, sb.slots, sb.len_after, d)
+        out = torch.empty((sb.n, H * dv), dtype=self.dtype, device=h.device)
+        if not sb.decode and mix_ops.diff_mfma_ok(self.dtype, sb.max_rows, d, dv, self.scale):
+            # matrix cores: both maps of a head in one workgroup, combined in the epilogue
+            mix_ops.attn_prefill_diff(out, p["q"], p["k"], p["v"], p.get("g"), sb.cu, H, G, d, dv, self.scale, self.softcap, self.span, self.mask, self.lam, self.diff,
+                                      self.eps, sb.max_rows)
+            return F.linear(out, self.w_o, self.b_o), p
         a = torch.empty((sb.n, H * M * dv), dtype=torch.float32, device=h.device)      # the maps' weighted sums stay float32 until they are combined
         if sb.decode:
             mix_ops.attn_decode_maps(a, p["q"], state["ring_k"], state["ring_v"], None, None, sb.slots, sb.len_after, H, M, self.scale, self.softcap, self.mask)
         else:
             mix_ops.attn_prefill_maps(a, p["q"], p["k"], p["v"], None, None, sb.cu, sb.tok_seq, sb.tok_pos, H, G, M, d, dv, self.scale, self.softcap, self.span,
                                       self.mask, max_rows=sb.max_rows)
-        out = torch.empty((sb.n, H * dv), dtype=self.dtype, device=h.device)
         mix_ops.diff_combine(out, a, self.lam, self.diff, self.eps, p.get("g"), H, dv)
         return F.linear(out, self.w_o, self.b_o), p
 

@@ -219,6 +219,14 @@ int exl3_mix_attn_decode_ex(void* out, int out_f32, const void* q, int64_t q_ld,
                             const void* gate, int64_t gate_ld, const float* sink, const int32_t* slots, const int32_t* len_after,
                             int n, int heads, int kv_heads, int maps, int dim, int vdim, float scale, float softcap, int window, int mask, int dtype, void* stream);
 
+/* Differential attention of a prompt step on the matrix cores, bfloat16 only: both maps of a head in one workgroup (the value tile is staged once for both)
+ * and the combination in the epilogue: out[n][h] = rms_unit(a1 - lambda a2) (1 - diff) sigmoid(gate[n][h]) (exl3_mix_diff_combine), with a1 / a2 the
+ * head's two attention maps (queries [n][heads][2][dim], keys [n][kv_heads][2][dim], values [n][kv_heads][vdim]) kept in float32 registers.
+ * dim <= 128, vdim <= 256, scale > 0. */
+int exl3_mix_attn_prefill_mfma_diff(void* out, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v, int64_t v_ld,
+                                    const void* gate, int64_t gate_ld, const int32_t* cu, int batch, int max_rows, int heads, int kv_heads, int dim, int vdim,
+                                    float scale, float softcap, int window, int mask, float lambda, float diff, float eps, void* stream);
+
 /* Queries and keys before the attention core, in place: per (row, head) RMS norm over dim with the weight q_norm / k_norm [dim] (NULL: none), then rotary
  * positions on the first rot_dims entries (freq [rot_dims / 2], NULL: none): pairs (i, i + rot_dims/2), or (2i, 2i+1) when `interleaved`; angle =
  * tok_pos * freq[i], cos and sin times `mag`.  q_heads and k_heads count every (head, map).  Keys and values of the rows with tok_pos >= len_after - window

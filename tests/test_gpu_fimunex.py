@@ -292,6 +292,26 @@ def test_chunked_two_map_attention_prompt(gpu, dtype, mfma, H, G, d, dv, span, s
         assert rel(out, torch.cat(want)) < TOL[dtype]
 
 
+@pytest.mark.parametrize("H,G,d,dv,span,softcap", [(4, 2, 16, 24, 9, 7.0), (2, 2, 8, 8, 1, 0.0), (3, 1, 12, 10, 64, 3.0), (2, 1, 40, 72, 130, 0.0), (2, 1, 128, 256, 100, 30.0),
+                                                   (2, 2, 64, 128, 200, 0.0)])
+def test_two_maps_and_their_combination_in_one_kernel(gpu, H, G, d, dv, span, softcap):
+    """The matrix-core kernel that keeps both maps of a head in one workgroup and combines them in its epilogue, against the oracle's maps combined in
+    float64 -- among them a dominant key just inside and just outside a chunk's start."""
+    from exllamav3_amd import mix_ops
+    lens = [150, 1, 37, 2, 300]
+    for spike in (None, (4, 2 * span + 3, 2 * span) if 2 * span + 3 < 300 else None, (4, 2 * span + 3, 2 * span - 1) if 2 * span + 3 < 300 else None):
+        q, k, v, want = _attention_case(gpu, torch.bfloat16, H, G, d, dv, span, softcap, lens, 17, spike=spike)
+        g = torch.Generator().manual_seed(3)
+        gate = torch.randn(sum(lens), H, generator=g).to(torch.bfloat16)
+        lam, diff = 0.77, 0.3
+        a = torch.cat(want).reshape(-1, H, 2, dv)
+        truth_out = (fo.rms_unit(a[:, :, 0] - lam * a[:, :, 1], 1e-5) * (1.0 - diff) * torch.sigmoid(gate.to(F64))[:, :, None]).reshape(-1, H * dv)
+        cu, seq, pos, sl, p0, la = batch_tensors(gpu, lens)
+        out = torch.empty((sum(lens), H * dv), dtype=torch.bfloat16, device=gpu)
+        mix_ops.attn_prefill_diff(out, q.to(gpu), k.to(gpu), v.to(gpu), gate.to(gpu), cu, H, G, d, dv, 0.4, softcap, span, mix_ops.MASK_CHUNK, lam, diff, 1e-5, max(lens))
+        assert rel(out, truth_out) < TOL[torch.bfloat16], spike
+
+
 @pytest.mark.parametrize("dtype,mfma", [(torch.float32, False), (torch.bfloat16, True)])
 @pytest.mark.parametrize("edge", ["inside", "outside"])
 def test_a_dominant_key_at_the_chunk_edge_in_a_prompt(gpu, dtype, mfma, edge):
