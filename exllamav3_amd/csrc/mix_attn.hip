@@ -38,7 +38,7 @@ __global__ __launch_bounds__(64) void attn_store_kernel(T* __restrict__ v_norm, 
 
 // `maps` attention maps per head (differential attention: 2): queries are laid out [head][map][dim], keys [kv head][map][dim], every map of a head reads
 // the values of the head's key/value head, and the result is [row][head][map][vdim].  mask 0: the last `window` positions; 1: the positions of the row's
-// own chunk of `window` positions (chunks counted from position 0).
+// own chunk of `window` positions (a chunk starts where the position is a multiple of `window`).
 template <typename T, int MAXV, typename TO>
 __global__ __launch_bounds__(64 * AT_WAVES) void attn_prefill_kernel(TO* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ k, int64_t k_ld,
                                                           const T* __restrict__ v, int64_t v_ld, const T* __restrict__ gate, int64_t gate_ld, const float* __restrict__ sink,

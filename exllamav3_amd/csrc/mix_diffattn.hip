@@ -77,6 +77,89 @@ __global__ __launch_bounds__(64 * QP_WAVES) void qk_prep_kernel(T* __restrict__ 
     }
 }
 
+// The same for rows that fit the LDS and allow 16-byte accesses (dim and vdim multiples of VN = 16 / sizeof(T) elements, 16-byte aligned blocks and rings):
+// the workgroup loads the row's queries and keys with 16 bytes per lane into LDS (float32), a wave per vector norms and rotates there, and the
+// workgroup stores 16 bytes per lane -- queries and keys in place, keys and values into the rings.  LDS: (q_heads + k_heads) * dim + rot_dims floats.
+template <typename T> struct qvec;
+template <> struct qvec<bf16_t> { static constexpr int N = 8; };
+template <> struct qvec<float> { static constexpr int N = 4; };
+
+template <typename T>
+__global__ __launch_bounds__(64 * QP_WAVES) void qk_prep_row_kernel(T* __restrict__ q, int64_t q_ld, T* __restrict__ k, int64_t k_ld, const T* __restrict__ v, int64_t v_ld,
+                                                         const float* __restrict__ q_norm, const float* __restrict__ k_norm, const float* __restrict__ freq, int rot_dims,
+                                                         float mag, int interleaved, float eps, T* __restrict__ ring_k, T* __restrict__ ring_v,
+                                                         const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ slots,
+                                                         const int32_t* __restrict__ len_after, int q_heads, int k_heads, int v_heads, int dim, int vdim, int window)
+{
+    constexpr int VN = qvec<T>::N;
+    extern __shared__ float smem[];                           // cos [rot_dims / 2] | sin [rot_dims / 2] | the row: q_heads * dim, k_heads * dim
+    const int n = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int half = freq ? rot_dims >> 1 : 0;
+    float* cs = smem;
+    float* sn = smem + half;
+    float* row = smem + 2 * half;
+    const int b = tok_seq[n], pos = tok_pos[n];
+    const bool keep = pos >= len_after[b] - window;
+    const int64_t ring_row = (int64_t) slots[b] * window + (pos % window);
+    const int nq = q_heads * dim, nk = k_heads * dim, nv = v_heads * vdim;
+    T* qr = q + (int64_t) n * q_ld;
+    T* kr = k + (int64_t) n * k_ld;
+    for (int i = threadIdx.x * VN; i < nq + nk; i += 64 * QP_WAVES * VN)
+    {
+        union { uint4 v; T e[VN]; } t;
+        t.v = *(const uint4*) (i < nq ? qr + i : kr + (i - nq));
+        #pragma unroll
+        for (int e = 0; e < VN; ++e) row[i + e] = to_f(t.e[e]);
+    }
+    if (keep)                                                 // values: straight into the ring
+    {
+        const T* vr = v + (int64_t) n * v_ld;
+        T* rv = ring_v + ring_row * nv;
+        for (int i = threadIdx.x * VN; i < nv; i += 64 * QP_WAVES * VN) *(uint4*) (rv + i) = *(const uint4*) (vr + i);
+    }
+    for (int p = threadIdx.x; p < half; p += 64 * QP_WAVES)
+    {
+        const float a = (float) pos * freq[p];
+        cs[p] = cosf(a) * mag; sn[p] = sinf(a) * mag;
+    }
+    __syncthreads();
+    for (int item = wv; item < q_heads + k_heads; item += QP_WAVES)
+    {
+        float* buf = row + item * dim;
+        const float* nw = item < q_heads ? q_norm : k_norm;
+        if (nw)
+        {
+            float ss = 0.f;
+            for (int i = lane; i < dim; i += 64) { const float x = buf[i]; ss += x * x; }
+            ss = wave_sum(ss);
+            const float inv = 1.0f / sqrtf(ss / (float) dim + eps);
+            for (int i = lane; i < dim; i += 64) buf[i] = buf[i] * inv * nw[i];
+            __builtin_amdgcn_wave_barrier();                  // LDS serves a wave's accesses in order: the stores above are visible to the reads below
+        }
+        for (int p = lane; p < half; p += 64)
+        {
+            const int i0 = interleaved ? 2 * p : p, i1 = interleaved ? 2 * p + 1 : p + half;
+            const float u = buf[i0], w = buf[i1], c = cs[p], s = sn[p];
+            buf[i0] = u * c - w * s;
+            buf[i1] = w * c + u * s;
+        }
+    }
+    __syncthreads();
+    T* rk = keep ? ring_k + ring_row * nk : nullptr;
+    for (int i = threadIdx.x * VN; i < nq + nk; i += 64 * QP_WAVES * VN)
+    {
+        union { uint4 v; T e[VN]; } t;
+        #pragma unroll
+        for (int e = 0; e < VN; ++e) t.e[e] = from_f<T>(row[i + e]);
+        if (i < nq) *(uint4*) (qr + i) = t.v;
+        else
+        {
+            *(uint4*) (kr + (i - nq)) = t.v;
+            if (rk) *(uint4*) (rk + (i - nq)) = t.v;
+        }
+    }
+}
+
 // a [n][heads][2][vdim] (float32): out[n][h * vdim + c] = o_c / sqrt(mean_c(o^2) + eps) * (1 - diff) * sigmoid(gate[n][h]), o = a[.,0] - lambda a[.,1]
 template <typename T>
 __global__ __launch_bounds__(64) void diff_combine_kernel(T* __restrict__ out, const float* __restrict__ a, float lambda, float diff, float eps, const T* __restrict__ gate,
@@ -105,6 +188,17 @@ extern "C" int exl3_mix_qk_prep(void* q, int64_t q_ld, void* k, int64_t k_ld, co
     MIX_CHECK(q_ld >= (int64_t) q_heads * dim && k_ld >= (int64_t) k_heads * dim && v_ld >= (int64_t) v_heads * vdim, "mix_qk_prep: bad row strides");
     MIX_CHECK(!freq || (rot_dims >= 2 && rot_dims % 2 == 0 && rot_dims <= dim), "mix_qk_prep: %d rotated entries of %d", rot_dims, dim);
     if (n == 0) return EXL3_MIX_OK;
+    const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
+    const size_t sm_row = (size_t) ((freq ? rot_dims : 0) + (int64_t) (q_heads + k_heads) * dim) * sizeof(float);
+    const bool by16 = dim % vn == 0 && vdim % vn == 0 && q_ld % vn == 0 && k_ld % vn == 0 && v_ld % vn == 0 && (uintptr_t) q % 16 == 0 && (uintptr_t) k % 16 == 0 &&
+                      (uintptr_t) v % 16 == 0 && (uintptr_t) ring_k % 16 == 0 && (uintptr_t) ring_v % 16 == 0 && sm_row <= 48 * 1024;
+    if (by16)
+    {
+        MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(qk_prep_row_kernel<T>, dim3(n), dim3(64 * QP_WAVES), sm_row, (hipStream_t) stream,
+                                                 (T*) q, q_ld, (T*) k, k_ld, (const T*) v, v_ld, q_norm, k_norm, freq, rot_dims, mag, interleaved, eps, (T*) ring_k, (T*) ring_v,
+                                                 tok_seq, tok_pos, slots, len_after, q_heads, k_heads, v_heads, dim, vdim, window));
+        return mix_check_launch("mix_qk_prep");
+    }
     const size_t sm = (size_t) ((freq ? rot_dims : 0) + QP_WAVES * dim) * sizeof(float);
     MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(qk_prep_kernel<T>, dim3(n), dim3(64 * QP_WAVES), sm, (hipStream_t) stream,
                                              (T*) q, q_ld, (T*) k, k_ld, (const T*) v, v_ld, q_norm, k_norm, freq, rot_dims, mag, interleaved, eps, (T*) ring_k, (T*) ring_v,

@@ -3,7 +3,7 @@ Fimunex: a decoder-only model of pre-norm blocks over a float32 stream whose sub
 differential attention (two attention maps per head over shared values, RMS-normed and rotated queries / keys, soft-capped scores, a chunk mask, a
 head-wise sigmoid gate); the feed-forward is a mixture of ungated relu^2 experts chosen by a softmax router with a selection-only correction, groups of
 experts of which only the best are eligible, and trailing router outputs that stand for experts which return their input -- or none.  A block of
-consecutive layers may run several times in a row with the same weights; each pass has its own state.  The order of layers and every size and constant
+consecutive layers may run several times in a row with the same weights, state being kept per pass.  The order of layers and every size and constant
 come from config.json:
 
     architecture "Fimunex"; vocab; width; norm.eps; canon.taps; logit_softcap (optional); loop {start, stop, times} (optional)

@@ -524,7 +524,7 @@ class CanonNorm:
         self.dtype = torch.bfloat16                                  # until load() says otherwise
 
     def load(self, stc, norm_key: str, conv_key: str, dtype, device):
-        self.w = (1.0 + _f32(stc, norm_key, device)).contiguous()              # the stored weight lies around zero
+        self.w = (1.0 + _f32(stc, norm_key, device)).contiguous()              # the checkpoint holds w, the norm multiplies by 1 + w
         self.conv = _f32(stc, conv_key, device).t().contiguous()               # stored [width, taps]; the kernels read one tap of neighbouring channels at once
         assert self.w.numel() == self.width and self.conv.shape == (self.taps, self.width)
         self.dtype = dtype

@@ -43,7 +43,7 @@ extern "C" {
 #define EXL3_MIX_ACT_SILU      2
 
 /* attention masks: WINDOW: a row sees the last `window` positions up to itself; CHUNK: the positions up to itself inside its own chunk of `window`
- * positions, chunks counted from position 0 of the sequence. */
+ * positions (a chunk starts where the sequence's position is a multiple of `window`). */
 #define EXL3_MIX_MASK_WINDOW 0
 #define EXL3_MIX_MASK_CHUNK  1
 

@@ -13,7 +13,7 @@ def rms_unit(x, eps):
 
 
 def norm_one_plus(x, w, eps):
-    """RMS norm whose stored weight lies around zero."""
+    """RMS norm with a one-plus weight: the checkpoint holds w, the norm multiplies by 1 + w."""
     return rms_unit(x, eps) * (1.0 + w)
 
 
@@ -61,7 +61,7 @@ def rotate_half(x, cos, sin, dims):
 
 
 def chunk_softmax_attention(q, k, v, scale, softcap, chunk):
-    """q [T, d], k [T, d], v [T, dv] of one map of one head: token i sees j <= i of its own chunk (chunks counted from position 0)."""
+    """q [T, d], k [T, d], v [T, dv] of one map of one head: token i sees j <= i with i // chunk == j // chunk, i and j being positions in the sequence."""
     T = q.shape[0]
     out = torch.zeros(T, v.shape[1], dtype=F64)
     for i in range(T):

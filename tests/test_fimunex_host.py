@@ -111,7 +111,7 @@ def test_config_defaults_and_refusals():
 
 
 def test_model_from_a_written_checkpoint_on_the_cpu(tmp_path):
-    """Loading needs no GPU: the tensors land where the mechanisms expect them, the norm weights are stored around zero and held as one plus, the state of
+    """Loading needs no GPU: the tensors land where the mechanisms expect them, the norm weights w of the checkpoint are held as 1 + w, the state of
     a looped layer exists once per pass."""
     from safetensors.torch import save_file
     from exllamav3_amd import registry

@@ -227,14 +227,15 @@ def test_norm_and_input_convolution_prompt_then_decode(gpu, dtype, taps):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_query_key_norm_rotation_and_ring_store(gpu, dtype):
+@pytest.mark.parametrize("H,G,d,dv,dims,pad", [(3, 1, 12, 10, 6, 5), (3, 1, 16, 24, 8, 8), (4, 2, 64, 128, 64, 0)])      # the last two: rows that allow 16-byte accesses
+def test_query_key_norm_rotation_and_ring_store(gpu, dtype, H, G, d, dv, dims, pad):
     from exllamav3_amd import mix_ops
     from exllamav3_amd.modules import rotary_frequencies
     g = torch.Generator().manual_seed(5)
-    H, G, d, dv, span, dims = 3, 1, 12, 10, 5, 6
+    span = 5
     lens = [7, 3]
     n = sum(lens)
-    wide = torch.randn(n, H * 2 * d + G * 2 * d + G * dv + 5, generator=g).to(dtype)
+    wide = torch.randn(n, H * 2 * d + G * 2 * d + G * dv + pad, generator=g).to(dtype)
     qn, kn = 1.0 + 0.3 * torch.randn(d, generator=g), 1.0 + 0.3 * torch.randn(d, generator=g)
     dev = wide.to(gpu)
     q, k, v = dev[:, :H * 2 * d], dev[:, H * 2 * d: (H + G) * 2 * d], dev[:, (H + G) * 2 * d: (H + G) * 2 * d + G * dv]
