@@ -39,8 +39,8 @@ __global__ __launch_bounds__(64) void attn_store_kernel(T* __restrict__ v_norm, 
 // `maps` attention maps per head (differential attention: 2): queries are laid out [head][map][dim], keys [kv head][map][dim], every map of a head reads
 // the values of the head's key/value head, and the result is [row][head][map][vdim].  mask 0: the last `window` positions; 1: the positions of the row's
 // own chunk of `window` positions (a chunk starts where the position is a multiple of `window`).
-template <typename T, int MAXV, typename TO>
-__global__ __launch_bounds__(64 * AT_WAVES) void attn_prefill_kernel(TO* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ k, int64_t k_ld,
+template <typename T, int MAXV, typename TO, int NW>
+__global__ __launch_bounds__(64 * NW) void attn_prefill_kernel(TO* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ k, int64_t k_ld,
                                                           const T* __restrict__ v, int64_t v_ld, const T* __restrict__ gate, int64_t gate_ld, const float* __restrict__ sink,
                                                           const int32_t* __restrict__ cu, const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
                                                           int heads, int kv_heads, int maps, int dim, int vdim, float scale, float softcap, int window, int mask)
@@ -53,15 +53,15 @@ __global__ __launch_bounds__(64 * AT_WAVES) void attn_prefill_kernel(TO* __restr
     const int lo = mask == EXL3_MIX_MASK_CHUNK ? (i / window) * window : max(0, i - window + 1);
     const float gt = gate ? sigmoid_f(to_f(gate[(int64_t) n * gate_ld + h])) : 1.0f;
     const T* kb = k + (int64_t) (first + lo) * k_ld + (int64_t) kh * dim;
-    attn_row<T, MAXV, TO>(out + ((int64_t) n * heads * maps + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim, q, dim, kb, k_ld,
+    attn_row<T, MAXV, TO, NW>(out + ((int64_t) n * heads * maps + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim, q, dim, kb, k_ld,
                           v + (int64_t) (first + lo) * v_ld + (int64_t) g * vdim, v_ld,
                           i - lo + 1, dim, vdim, scale, sink != nullptr, sink ? sink[h] : 0.f, gt, rows_are_16_byte(kb, k_ld, dim), smem, softcap);
 }
 
 // Rings: ring_k [slots][window][kv_heads * maps][dim], ring_v [slots][window][kv_heads][vdim], entry = position % window.  mask 0: the newest
 // min(len, window) entries (all of them, in any order); 1: the row's chunk, which is the entries 0 .. (len - 1) % window.
-template <typename T, int MAXV, typename TO>
-__global__ __launch_bounds__(64 * AT_WAVES) void attn_decode_kernel(TO* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ ring_k,
+template <typename T, int MAXV, typename TO, int NW>
+__global__ __launch_bounds__(64 * NW) void attn_decode_kernel(TO* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ ring_k,
                                                          const T* __restrict__ ring_v, const T* __restrict__ gate, int64_t gate_ld, const float* __restrict__ sink,
                                                          const int32_t* __restrict__ slots, const int32_t* __restrict__ len_after,
                                                          int heads, int kv_heads, int maps, int dim, int vdim, float scale, float softcap, int window, int mask)
@@ -74,7 +74,7 @@ __global__ __launch_bounds__(64 * AT_WAVES) void attn_decode_kernel(TO* __restri
     const int64_t row0 = (int64_t) slots[n] * window;
     const float gt = gate ? sigmoid_f(to_f(gate[(int64_t) n * gate_ld + h])) : 1.0f;
     const T* kb = ring_k + (row0 * kheads + kh) * dim;
-    attn_row<T, MAXV, TO>(out + ((int64_t) n * heads * maps + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim, q, dim,
+    attn_row<T, MAXV, TO, NW>(out + ((int64_t) n * heads * maps + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim, q, dim,
                           kb, (int64_t) kheads * dim, ring_v + (row0 * kv_heads + g) * vdim, (int64_t) kv_heads * vdim,
                           count, dim, vdim, scale, sink != nullptr, sink ? sink[h] : 0.f, gt, rows_are_16_byte(kb, (int64_t) kheads * dim, dim), smem, softcap);
 }
@@ -92,19 +92,22 @@ extern "C" int exl3_mix_attn_store(void* v_norm, void* ring_k, void* ring_v, con
     return mix_check_launch("mix_attn_store");
 }
 
-#define ATTN_LAUNCH_TO(KERNEL, TO, ...) \
+#define ATTN_LAUNCH_NW(KERNEL, TO, NWV, ...) \
     do { \
-        if (mv == 1)      hipLaunchKernelGGL((KERNEL<T, 1, TO>), dim3(n, heads * maps), dim3(64 * AT_WAVES), sm, (hipStream_t) stream, (TO*) out, __VA_ARGS__); \
-        else if (mv == 2) hipLaunchKernelGGL((KERNEL<T, 2, TO>), dim3(n, heads * maps), dim3(64 * AT_WAVES), sm, (hipStream_t) stream, (TO*) out, __VA_ARGS__); \
-        else if (mv <= 4) hipLaunchKernelGGL((KERNEL<T, 4, TO>), dim3(n, heads * maps), dim3(64 * AT_WAVES), sm, (hipStream_t) stream, (TO*) out, __VA_ARGS__); \
-        else              hipLaunchKernelGGL((KERNEL<T, 8, TO>), dim3(n, heads * maps), dim3(64 * AT_WAVES), sm, (hipStream_t) stream, (TO*) out, __VA_ARGS__); \
+        const size_t sm = (size_t) (dim + NWV * 64 + NWV * (2 + mvt * 64)) * sizeof(float); \
+        if (mv == 1)      hipLaunchKernelGGL((KERNEL<T, 1, TO, NWV>), dim3(n, heads * maps), dim3(64 * NWV), sm, (hipStream_t) stream, (TO*) out, __VA_ARGS__); \
+        else if (mv == 2) hipLaunchKernelGGL((KERNEL<T, 2, TO, NWV>), dim3(n, heads * maps), dim3(64 * NWV), sm, (hipStream_t) stream, (TO*) out, __VA_ARGS__); \
+        else if (mv <= 4) hipLaunchKernelGGL((KERNEL<T, 4, TO, NWV>), dim3(n, heads * maps), dim3(64 * NWV), sm, (hipStream_t) stream, (TO*) out, __VA_ARGS__); \
+        else              hipLaunchKernelGGL((KERNEL<T, 8, TO, NWV>), dim3(n, heads * maps), dim3(64 * NWV), sm, (hipStream_t) stream, (TO*) out, __VA_ARGS__); \
     } while (0)
+// `wide`: sixteen waves per (row, head) instead of four -- steps of few rows over long caches are bound by the chain of key chunks a wave walks, not by bytes
+#define ATTN_LAUNCH_TO(KERNEL, TO, ...) \
+    do { if (wide) ATTN_LAUNCH_NW(KERNEL, TO, 16, __VA_ARGS__); else ATTN_LAUNCH_NW(KERNEL, TO, AT_WAVES, __VA_ARGS__); } while (0)
 // the result in the activation type, or (out_f32) in float32
 #define ATTN_LAUNCH(KERNEL, ...) \
     do { \
         const int mv = (vdim + 63) / 64; \
         const int mvt = mv == 1 ? 1 : (mv == 2 ? 2 : (mv <= 4 ? 4 : 8)); \
-        const size_t sm = (size_t) (dim + AT_WAVES * 64 + AT_WAVES * (2 + mvt * 64)) * sizeof(float); \
         MIX_DISPATCH_T(dtype, if (out_f32) ATTN_LAUNCH_TO(KERNEL, float, __VA_ARGS__); else ATTN_LAUNCH_TO(KERNEL, T, __VA_ARGS__)); \
     } while (0)
 
@@ -126,6 +129,7 @@ extern "C" int exl3_mix_attn_prefill_ex(void* out, int out_f32, const void* q, i
     MIX_CHECK(q_ld >= (int64_t) heads * maps * dim && k_ld >= (int64_t) kv_heads * maps * dim && v_ld >= (int64_t) kv_heads * vdim && (!gate || gate_ld >= heads),
               "mix_attn_prefill: bad row strides");
     if (n == 0) return EXL3_MIX_OK;
+    const bool wide = false;
     ATTN_LAUNCH(attn_prefill_kernel, (const T*) q, q_ld, (const T*) k, k_ld, (const T*) v, v_ld, (const T*) gate, gate_ld, sink, cu, tok_seq, tok_pos,
                 heads, kv_heads, maps, dim, vdim, scale, softcap, window, mask);
     return mix_check_launch("mix_attn_prefill");
@@ -147,6 +151,7 @@ extern "C" int exl3_mix_attn_decode_ex(void* out, int out_f32, const void* q, in
     if (int rc = attn_check("mix_attn_decode", n, heads, kv_heads, maps, dim, vdim, window, mask, softcap, gate)) return rc;
     MIX_CHECK(q_ld >= (int64_t) heads * maps * dim && (!gate || gate_ld >= heads), "mix_attn_decode: bad row strides");
     if (n == 0) return EXL3_MIX_OK;
+    const bool wide = (int64_t) n * heads * maps <= 256 && window > 256 && vdim <= 256;
     ATTN_LAUNCH(attn_decode_kernel, (const T*) q, q_ld, (const T*) ring_k, (const T*) ring_v, (const T*) gate, gate_ld, sink, slots, len_after,
                 heads, kv_heads, maps, dim, vdim, scale, softcap, window, mask);
     return mix_check_launch("mix_attn_decode");

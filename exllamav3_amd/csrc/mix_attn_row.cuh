@@ -3,8 +3,8 @@
 #pragma once
 #include "mix_common.cuh"
 
-// One workgroup of AT_WAVES waves per (row, query head).  Keys kb + j * k_step, values vb + j * v_step, j < count: wave w takes the 64-key chunks
-// w, w + AT_WAVES, ... (one key per lane, its row read in 16-byte pieces when the layout allows), keeps its own running maximum, sum and
+// One workgroup of NW waves (AT_WAVES unless the caller asks for more: few rows, long caches) per (row, query head).  Keys kb + j * k_step, values vb + j * v_step, j < count: wave w takes the 64-key chunks
+// w, w + NW, ... (one key per lane, its row read in 16-byte pieces when the layout allows), keeps its own running maximum, sum and
 // value accumulators (MAXV = ceil(vdim / 64) per lane), and the waves are merged through LDS at the end.  Wave 0 starts from the sink.
 // The query's first dim1 elements are read from q, the rest from q2 (dim1 = dim: one part).  softcap > 0: score <- softcap tanh(score / softcap).
 // TO: the element type of the result (float keeps the weighted sum unrounded for a caller that combines several maps).
@@ -14,16 +14,16 @@ template <typename T> struct kvec;
 template <> struct kvec<bf16_t> { static constexpr int N = 8; };
 template <> struct kvec<float> { static constexpr int N = 4; };
 
-template <typename T, int MAXV, typename TO = T>
+template <typename T, int MAXV, typename TO = T, int NW = AT_WAVES>
 __device__ __forceinline__ void attn_row(TO* __restrict__ out, const T* __restrict__ q, const T* q2, int dim1, const T* __restrict__ kb, int64_t k_step, const T* __restrict__ vb,
                                          int64_t v_step, int count, int dim, int vdim, float scale, bool has_sink, float sink, float gate, bool k_vec,
                                          float* smem, float softcap = 0.f)
 {
     float* qs = smem;                                   // [dim]
-    float* ps = qs + dim;                               // [AT_WAVES][64]
-    float* mg = ps + AT_WAVES * 64;                     // [AT_WAVES][2 + MAXV * 64]: m, l, accumulators
+    float* ps = qs + dim;                               // [NW][64]
+    float* mg = ps + NW * 64;                     // [NW][2 + MAXV * 64]: m, l, accumulators
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    for (int i = threadIdx.x; i < dim; i += 64 * AT_WAVES) qs[i] = to_f(i < dim1 ? q[i] : q2[i - dim1]);      // the query may come in two parts
+    for (int i = threadIdx.x; i < dim; i += 64 * NW) qs[i] = to_f(i < dim1 ? q[i] : q2[i - dim1]);      // the query may come in two parts
     __syncthreads();
     const bool seeded = has_sink && w == 0;
     float m = seeded ? sink : -INFINITY, l = seeded ? 1.0f : 0.0f;
@@ -32,7 +32,7 @@ __device__ __forceinline__ void attn_row(TO* __restrict__ out, const T* __restri
     for (int i = 0; i < MAXV; ++i) acc[i] = 0.f;
     float* pw = ps + w * 64;
     constexpr int VN = kvec<T>::N;
-    for (int j0 = w * 64; j0 < count; j0 += 64 * AT_WAVES)
+    for (int j0 = w * 64; j0 < count; j0 += 64 * NW)
     {
         const int j = j0 + lane;
         float s = -INFINITY;
@@ -94,12 +94,12 @@ __device__ __forceinline__ void attn_row(TO* __restrict__ out, const T* __restri
     if (w != 0) return;
     float mt = -INFINITY;
     #pragma unroll
-    for (int ww = 0; ww < AT_WAVES; ++ww) mt = fmaxf(mt, mg[ww * (2 + MAXV * 64)]);
+    for (int ww = 0; ww < NW; ++ww) mt = fmaxf(mt, mg[ww * (2 + MAXV * 64)]);
     float lt = 0.f;
     #pragma unroll
     for (int i = 0; i < MAXV; ++i) acc[i] = 0.f;
     #pragma unroll
-    for (int ww = 0; ww < AT_WAVES; ++ww)
+    for (int ww = 0; ww < NW; ++ww)
     {
         const float* o = mg + ww * (2 + MAXV * 64);
         const float f = (o[0] == -INFINITY) ? 0.f : expf(o[0] - mt);

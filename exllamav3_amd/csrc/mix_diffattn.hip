@@ -84,8 +84,8 @@ template <typename T> struct qvec;
 template <> struct qvec<bf16_t> { static constexpr int N = 8; };
 template <> struct qvec<float> { static constexpr int N = 4; };
 
-template <typename T>
-__global__ __launch_bounds__(64 * QP_WAVES) void qk_prep_row_kernel(T* __restrict__ q, int64_t q_ld, T* __restrict__ k, int64_t k_ld, const T* __restrict__ v, int64_t v_ld,
+template <typename T, int QR_WAVES>
+__global__ __launch_bounds__(64 * QR_WAVES) void qk_prep_row_kernel(T* __restrict__ q, int64_t q_ld, T* __restrict__ k, int64_t k_ld, const T* __restrict__ v, int64_t v_ld,
                                                          const float* __restrict__ q_norm, const float* __restrict__ k_norm, const float* __restrict__ freq, int rot_dims,
                                                          float mag, int interleaved, float eps, T* __restrict__ ring_k, T* __restrict__ ring_v,
                                                          const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ slots,
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(64 * QP_WAVES) void qk_prep_row_kernel(T* __restric
     const int nq = q_heads * dim, nk = k_heads * dim, nv = v_heads * vdim;
     T* qr = q + (int64_t) n * q_ld;
     T* kr = k + (int64_t) n * k_ld;
-    for (int i = threadIdx.x * VN; i < nq + nk; i += 64 * QP_WAVES * VN)
+    for (int i = threadIdx.x * VN; i < nq + nk; i += 64 * QR_WAVES * VN)
     {
         union { uint4 v; T e[VN]; } t;
         t.v = *(const uint4*) (i < nq ? qr + i : kr + (i - nq));
@@ -115,15 +115,16 @@ __global__ __launch_bounds__(64 * QP_WAVES) void qk_prep_row_kernel(T* __restric
     {
         const T* vr = v + (int64_t) n * v_ld;
         T* rv = ring_v + ring_row * nv;
-        for (int i = threadIdx.x * VN; i < nv; i += 64 * QP_WAVES * VN) *(uint4*) (rv + i) = *(const uint4*) (vr + i);
+        for (int i = threadIdx.x * VN; i < nv; i += 64 * QR_WAVES * VN) *(uint4*) (rv + i) = *(const uint4*) (vr + i);
     }
-    for (int p = threadIdx.x; p < half; p += 64 * QP_WAVES)
+    for (int p = threadIdx.x; p < half; p += 64 * QR_WAVES)
     {
-        const float a = (float) pos * freq[p];
-        cs[p] = cosf(a) * mag; sn[p] = sinf(a) * mag;
+        float sv, cv;
+        sincosf((float) pos * freq[p], &sv, &cv);
+        cs[p] = cv * mag; sn[p] = sv * mag;
     }
     __syncthreads();
-    for (int item = wv; item < q_heads + k_heads; item += QP_WAVES)
+    for (int item = wv; item < q_heads + k_heads; item += QR_WAVES)
     {
         float* buf = row + item * dim;
         const float* nw = item < q_heads ? q_norm : k_norm;
@@ -146,7 +147,7 @@ __global__ __launch_bounds__(64 * QP_WAVES) void qk_prep_row_kernel(T* __restric
     }
     __syncthreads();
     T* rk = keep ? ring_k + ring_row * nk : nullptr;
-    for (int i = threadIdx.x * VN; i < nq + nk; i += 64 * QP_WAVES * VN)
+    for (int i = threadIdx.x * VN; i < nq + nk; i += 64 * QR_WAVES * VN)
     {
         union { uint4 v; T e[VN]; } t;
         #pragma unroll
@@ -194,9 +195,13 @@ extern "C" int exl3_mix_qk_prep(void* q, int64_t q_ld, void* k, int64_t k_ld, co
                       (uintptr_t) v % 16 == 0 && (uintptr_t) ring_k % 16 == 0 && (uintptr_t) ring_v % 16 == 0 && sm_row <= 48 * 1024;
     if (by16)
     {
-        MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(qk_prep_row_kernel<T>, dim3(n), dim3(64 * QP_WAVES), sm_row, (hipStream_t) stream,
-                                                 (T*) q, q_ld, (T*) k, k_ld, (const T*) v, v_ld, q_norm, k_norm, freq, rot_dims, mag, interleaved, eps, (T*) ring_k, (T*) ring_v,
-                                                 tok_seq, tok_pos, slots, len_after, q_heads, k_heads, v_heads, dim, vdim, window));
+        // few rows (steps of one row per sequence): sixteen waves share a row's vectors, the step is bound by the chain a wave walks; many rows: four
+        #define QR_LAUNCH(NWV) \
+            MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((qk_prep_row_kernel<T, NWV>), dim3(n), dim3(64 * NWV), sm_row, (hipStream_t) stream, \
+                                                     (T*) q, q_ld, (T*) k, k_ld, (const T*) v, v_ld, q_norm, k_norm, freq, rot_dims, mag, interleaved, eps, (T*) ring_k, (T*) ring_v, \
+                                                     tok_seq, tok_pos, slots, len_after, q_heads, k_heads, v_heads, dim, vdim, window))
+        if (n <= 64) QR_LAUNCH(16); else QR_LAUNCH(4);
+        #undef QR_LAUNCH
         return mix_check_launch("mix_qk_prep");
     }
     const size_t sm = (size_t) ((freq ? rot_dims : 0) + QP_WAVES * dim) * sizeof(float);
