@@ -15,7 +15,8 @@ from .mixer_bench import PEAK_BF16, PEAK_HBM, SIZES, TensorDict, _time, kernel_l
 # differential attention at the sizes of mixer_bench.SIZES: half the heads, each with two maps of the head dim and values twice as wide, so that the
 # projections and the attention core do the work of the plain attention layer of the same name; chunk = that layer's window
 TAPS = 4
-YARN = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+YARN = {"factor": 8.0, "original": 8192, "fast": 24.0, "slow": 2.0}
+SOFTCAP, DIFF, ROT_BASE = 30.0, 0.5, 1.0e6
 KINDS = [("attention", "none"), ("attention", "moe")]
 
 
@@ -44,8 +45,8 @@ def synth(size: dict, kinds, vocab=32000, seed=0, device="cuda:0", loop=None):
         vec(p + "mix.q.norm", d, 1.0); vec(p + "mix.k.norm", d, 1.0)
         for nm in ("lq1", "lk1", "lq2", "lk2"):
             vec(p + "mix." + nm, d)
-        mixer = {"heads": H, "kv_heads": G, "dim": d, "vdim": dv, "scale": d ** -0.5, "softcap": 50.0, "diff": 0.6, "mask": {"size": sh["chunk"]},
-                 "rot": {"base": 500000.0, "dims": d, "scaling": YARN}}
+        mixer = {"heads": H, "kv_heads": G, "dim": d, "vdim": dv, "scale": d ** -0.5, "softcap": SOFTCAP, "diff": DIFF, "mask": {"size": sh["chunk"]},
+                 "rot": {"base": ROT_BASE, "dims": d, "scaling": YARN}}
         if ff == "none":
             mlp = None
         else:
@@ -56,7 +57,7 @@ def synth(size: dict, kinds, vocab=32000, seed=0, device="cuda:0", loop=None):
             lin(p + "mlp.router", E + sh["identity"], w); vec(p + "mlp.correction", E + sh["identity"])
             mlp = {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": E, "top": top, "identity": sh["identity"], "groups": {"count": sh["groups"][0], "keep": sh["groups"][1]}}}
         layers.append({"type": mix, "mixer": mixer, "mlp": mlp})
-    cfg = {"architecture": "Fimunex", "vocab": vocab, "width": w, "norm": {"eps": 1e-5}, "canon": {"taps": TAPS}, "logit_softcap": 30.0, "layers": layers}
+    cfg = {"architecture": "Fimunex", "vocab": vocab, "width": w, "norm": {"eps": 1e-5}, "canon": {"taps": TAPS}, "logit_softcap": 20.0, "layers": layers}
     if loop:
         cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
     return cfg, TensorDict(t)
@@ -82,7 +83,7 @@ def diff_kernel_legs(size_name: str, prompt: int, ctx: int, dev):
     cu, seq, pos = i32([0, n]), torch.zeros(n, dtype=torch.int32, device=dev), torch.arange(n, dtype=torch.int32, device=dev)
     sl, la, p0 = i32([0]), i32([n]), i32([0])
     hbm = lambda by, t: {"us": t * 1e6, "GBps": by / t / 1e9, "of_hbm": by / t / PEAK_HBM}
-    freq, mag = rotary_frequencies(d, 500000.0, YARN)
+    freq, mag = rotary_frequencies(d, ROT_BASE, YARN)
     freq = freq.to(dev)
     q, k, v = rnd(n, H * 2 * d), rnd(n, G * 2 * d), rnd(n, G * dv)
     rk, rv = torch.zeros((16, C, G * 2, d), dtype=bf, device=dev), torch.zeros((16, C, G, dv), dtype=bf, device=dev)
@@ -92,26 +93,26 @@ def diff_kernel_legs(size_name: str, prompt: int, ctx: int, dev):
     a = torch.empty((n, H * 2 * dv), dtype=torch.float32, device=dev)
     pairs = sum(i % C + 1 for i in range(n))
     fl = 2.0 * (d + dv) * pairs * H * 2
-    for cap in (50.0, 0.0):
+    for cap in (SOFTCAP, 0.0):
         t = _time(lambda: mix_ops.attn_prefill_maps(a, q, k, v, None, None, cu, seq, pos, H, G, 2, d, dv, d ** -0.5, cap, C, mix_ops.MASK_CHUNK, max_rows=n, mfma=True), 10)
         out["attn_prefill_mfma_two_maps_chunk" + ("_softcap" if cap else "_no_softcap")] = {"ms": t * 1e3, "tflops": fl / t / 1e12, "of_bf16_peak": fl / t / PEAK_BF16}
     o, gt = torch.empty((n, H * dv), dtype=bf, device=dev), rnd(n, H)
-    for cap in (50.0, 0.0):
-        t = _time(lambda: mix_ops.attn_prefill_diff(o, q, k, v, gt, cu, H, G, d, dv, d ** -0.5, cap, C, mix_ops.MASK_CHUNK, 0.7, 0.6, 1e-5, n), 10)
+    for cap in (SOFTCAP, 0.0):
+        t = _time(lambda: mix_ops.attn_prefill_diff(o, q, k, v, gt, cu, H, G, d, dv, d ** -0.5, cap, C, mix_ops.MASK_CHUNK, 0.7, DIFF, 1e-5, n), 10)
         out["attn_prefill_mfma_diff_fused" + ("_softcap" if cap else "_no_softcap")] = {"ms": t * 1e3, "tflops": fl / t / 1e12, "of_bf16_peak": fl / t / PEAK_BF16}
-    t = _time(lambda: mix_ops.diff_combine(o, a, 0.7, 0.6, 1e-5, gt, H, dv), 20)
+    t = _time(lambda: mix_ops.diff_combine(o, a, 0.7, DIFF, 1e-5, gt, H, dv), 20)
     out["diff_combine_prefill"] = hbm(n * H * dv * (2 * 4 + 2), t)
     for bs in (1, 16):
         qd, ad = rnd(bs, H * 2 * d), torch.empty((bs, H * 2 * dv), dtype=torch.float32, device=dev)
         sld, lad = torch.arange(bs, dtype=torch.int32, device=dev), i32([ctx] * bs)
-        t = _time(lambda: mix_ops.attn_decode_maps(ad, qd, rk, rv, None, None, sld, lad, H, 2, d ** -0.5, 50.0, mix_ops.MASK_CHUNK), 50)
+        t = _time(lambda: mix_ops.attn_decode_maps(ad, qd, rk, rv, None, None, sld, lad, H, 2, d ** -0.5, SOFTCAP, mix_ops.MASK_CHUNK), 50)
         keys = (ctx - 1) % C + 1
         out[f"attn_decode_two_maps_bs{bs}"] = hbm(bs * keys * (G * 2 * d + G * dv) * 2, t)
         kd, vd, sq, pd = rnd(bs, G * 2 * d), rnd(bs, G * dv), torch.arange(bs, dtype=torch.int32, device=dev), i32([ctx - 1] * bs)
         t = _time(lambda: mix_ops.qk_prep(qd, kd, vd, qn, qn, freq, mag, False, 1e-5, rk, rv, sq, pd, sld, lad, d), 50)
         out[f"qk_prep_bs{bs}"] = {"us": t * 1e6}
         od, gd = torch.empty((bs, H * dv), dtype=bf, device=dev), rnd(bs, H)
-        t = _time(lambda: mix_ops.diff_combine(od, ad, 0.7, 0.6, 1e-5, gd, H, dv), 50)
+        t = _time(lambda: mix_ops.diff_combine(od, ad, 0.7, DIFF, 1e-5, gd, H, dv), 50)
         out[f"diff_combine_bs{bs}"] = {"us": t * 1e6}
     x, y, nw, cw = torch.randn(n, w, device=dev), rnd(n, w), torch.ones(w, device=dev), 0.3 * torch.randn(TAPS, w, device=dev)
     hn, h, ring = torch.empty((n, w), dtype=bf, device=dev), torch.empty((n, w), dtype=bf, device=dev), torch.zeros((16, TAPS - 1, w), dtype=bf, device=dev)
