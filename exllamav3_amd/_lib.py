@@ -236,7 +236,7 @@ def _declare(l):
 # ---- the sequence-mixer library (include/exl3_mix.h, csrc/mix_*.hip) -------------------------------------------------------------
 MIX_LIB_PATH = os.path.join(_HERE, "libexl3_mix.so")
 MIX_HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "exl3_mix.h")
-MIX_ABI_VERSION = 3
+MIX_ABI_VERSION = 4
 _mix = None
 
 
@@ -340,3 +340,17 @@ def _declare_mix(l):
     sig("exl3_mix_moe_combine_id", vp, vp, vp, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp)
     sig("exl3_mix_softcap", vp, i64, f32, vp)
     sig("exl3_mix_attn_prefill_mfma_diff", vp, vp, i64, vp, i64, vp, i64, vp, i64, vp, i32, i32, i32, i32, i32, i32, f32, f32, i32, i32, f32, f32, f32, vp)
+    sig("exl3_mix_embed_sinusoid", vp, vp, vp, vp, vp, f32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_layer_norm_rows", vp, vp, vp, vp, vp, f32, i32, i32, i32, vp)
+    sig("exl3_mix_residual_norm_conv", vp, vp, i64, vp, i64, f32, i32, i32, vp, vp, f32, vp, i64, vp, i64, vp, i32, vp, vp, vp, vp, i32, i32, i32, vp)
+    sig("exl3_mix_glu_act_rowgate", vp, vp, i64, vp, i64, vp, i64, i32, i32, i32, f32, i32, vp)
+    sig("exl3_mix_topk_grouped_ex", vp, vp, vp, vp, vp, i32, f32, i32, i32, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_paged_store", vp, vp, vp, i64, vp, i64, vp, i64, i32, vp, vp, vp, i32, i32, i32, i32, vp)
+    sig("exl3_mix_sigattn_prefill", vp, vp, i64, vp, i64, vp, i64, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, vp)
+    sig("exl3_mix_sigattn_decode", vp, vp, i64, vp, vp, vp, vp, i64, i32, vp, vp, i32, i32, i32, i32, i32, f32, i32, vp)
+    sig("exl3_mix_sigattn_prefill_mfma", vp, vp, i64, vp, i64, vp, i64, vp, vp, i32, i32, i32, i32, i32, i32, f32, vp)
+    sig("exl3_mix_mlstm_scan", vp, vp, vp, vp, vp, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, f32, i32, vp)
+    sig("exl3_mix_delta_prep", vp, vp, vp, vp, vp, vp, i64, vp, i32, vp, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, vp)
+    sig("exl3_mix_delta_scan", vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_head_norm_gate", vp, vp, vp, i32, vp, i64, i32, f32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_rms_pair", vp, vp, i64, vp, vp, i64, vp, f32, f32, i32, i32, i32, vp)

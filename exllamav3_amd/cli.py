@@ -72,7 +72,7 @@ def main(argv=None) -> int:
     t.add_argument("--model", required=True)
     t.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     t.add_argument("--out", required=True)
-    t.add_argument("--max-tokens", type=int, default=0, help="most tokens alive at once (slots are bounded per sequence; accepted and not needed)")
+    t.add_argument("--max-tokens", type=int, default=0, help="most tokens alive at once: sizes the pages of a model whose cache grows with its sequences")
     args = ap.parse_args(argv)
 
     if args.cmd == "models":
@@ -91,7 +91,7 @@ def main(argv=None) -> int:
         from .trace import TraceSession
         os.makedirs(args.out, exist_ok=True)
         model = _load(args)
-        TraceSession(model, args.out).run(sys.stdin)
+        TraceSession(model, args.out, args.max_tokens).run(sys.stdin)
         return 0
     return 2
 

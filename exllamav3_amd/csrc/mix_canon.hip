@@ -33,9 +33,14 @@ template <typename T> __device__ __forceinline__ float rounded(float v) { return
 // mode 0: x stays; 1: x += y; 2: x = y.  Then hn = x / sqrt(mean(x^2) + eps) * w.  With conv_w [taps][width] (one row per sequence, predecessors in the
 // ring): h = hn + sum_j conv_w[j][c] * (j == taps - 1 ? hn : ring[(pos - (taps - 1 - j)) % (taps - 1)]), positions below 0 count as zero rows, and hn goes
 // into the ring at pos % (taps - 1).  Without conv_w, h = hn.  V: elements per thread and access (4 when the rows allow it).
-template <typename T, int V>
-__global__ __launch_bounds__(CN_THREADS) void residual_rms_kernel(float* __restrict__ x, const T* __restrict__ y, int64_t y_ld, int mode, const float* __restrict__ w, float eps,
-                                                                  T* __restrict__ h, int64_t h_ld, const float* __restrict__ conv_w, int taps, T* __restrict__ ring,
+// CENTER: the norm is a layer norm, (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + bias, the mean taken first and the deviations squared after it.
+// y2 (optional): a second addend, y' = (y + y2) * y_scale (the two sublayers of a parallel block and the block's residual factor); without it y' = y * y_scale.
+// hn_out (optional): the normed row itself, for a consumer that reads it without the convolution.
+template <typename T, int V, bool CENTER>
+__global__ __launch_bounds__(CN_THREADS) void residual_rms_kernel(float* __restrict__ x, const T* __restrict__ y, int64_t y_ld, const T* __restrict__ y2, int64_t y2_ld, float y_scale,
+                                                                  int mode, const float* __restrict__ w, const float* __restrict__ bias, float eps,
+                                                                  T* __restrict__ h, int64_t h_ld, T* __restrict__ hn_out, int64_t hn_ld,
+                                                                  const float* __restrict__ conv_w, int taps, T* __restrict__ ring,
                                                                   const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
                                                                   const int32_t* __restrict__ slots, int width)
 {
@@ -43,6 +48,7 @@ __global__ __launch_bounds__(CN_THREADS) void residual_rms_kernel(float* __restr
     const int n = blockIdx.x;
     float* xr = x + (int64_t) n * width;
     const T* yr = y + (int64_t) n * y_ld;
+    const T* y2r = y2 ? y2 + (int64_t) n * y2_ld : nullptr;
     float ss = 0.f;
     for (int i = threadIdx.x * V; i < width; i += CN_THREADS * V)
     {
@@ -52,15 +58,34 @@ __global__ __launch_bounds__(CN_THREADS) void residual_rms_kernel(float* __restr
         {
             float a[V];
             if constexpr (V == 4) load4<T>(yr + i, (float (&)[4]) a); else a[0] = to_f(yr[i]);
+            if (y2r)
+            {
+                float a2[V];
+                if constexpr (V == 4) load4<T>(y2r + i, (float (&)[4]) a2); else a2[0] = to_f(y2r[i]);
+                #pragma unroll
+                for (int e = 0; e < V; ++e) a[e] += a2[e];
+            }
             #pragma unroll
-            for (int e = 0; e < V; ++e) v[e] = mode == 1 ? v[e] + a[e] : a[e];
+            for (int e = 0; e < V; ++e) v[e] = mode == 1 ? v[e] + a[e] * y_scale : a[e] * y_scale;
             if constexpr (V == 4) *(float4*) (xr + i) = make_float4(v[0], v[1], v[2], v[V - 1]); else xr[i] = v[0];
         }
         #pragma unroll
-        for (int e = 0; e < V; ++e) ss += v[e] * v[e];
+        for (int e = 0; e < V; ++e) ss += CENTER ? v[e] : v[e] * v[e];
     }
-    if (!h) return;
+    if (!h && !hn_out) return;
     ss = block_sum<CN_WAVES>(ss, red);
+    float mean = 0.f;
+    if constexpr (CENTER)
+    {
+        mean = ss / (float) width;
+        float dd = 0.f;
+        for (int i = threadIdx.x * V; i < width; i += CN_THREADS * V)                 // the thread's own part of x once more
+        {
+            #pragma unroll
+            for (int e = 0; e < V; ++e) { const float d = xr[i + e] - mean; dd += d * d; }
+        }
+        ss = block_sum<CN_WAVES>(dd, red);
+    }
     const float inv = 1.0f / sqrtf(ss / (float) width + eps);
     T* hr = h + (int64_t) n * h_ld;
     const int pos = conv_w ? tok_pos[n] : 0, keep = taps - 1;
@@ -74,8 +99,22 @@ __global__ __launch_bounds__(CN_THREADS) void residual_rms_kernel(float* __restr
             hn[0] = t.x; hn[1] = t.y; hn[2] = t.z; hn[V - 1] = t.w; wv[0] = u.x; wv[1] = u.y; wv[2] = u.z; wv[V - 1] = u.w;
         }
         else { hn[0] = xr[i]; wv[0] = w[i]; }
-        #pragma unroll
-        for (int e = 0; e < V; ++e) hn[e] = rounded<T>(hn[e] * inv * wv[e]);            // the normed row is held in the activation type wherever it is kept
+        if constexpr (CENTER)
+        {
+            #pragma unroll
+            for (int e = 0; e < V; ++e) hn[e] = rounded<T>((hn[e] - mean) * inv * wv[e] + (bias ? bias[i + e] : 0.f));
+        }
+        else
+        {
+            #pragma unroll
+            for (int e = 0; e < V; ++e) hn[e] = rounded<T>(hn[e] * inv * wv[e]);        // the normed row is held in the activation type wherever it is kept
+        }
+        if (hn_out)
+        {
+            T* dsth = hn_out + (int64_t) n * hn_ld + i;
+            if constexpr (V == 4) store4<T>(dsth, (const float (&)[4]) hn); else dsth[0] = from_f<T>(hn[0]);
+        }
+        if (!h) continue;
         if (!conv_w)
         {
             if constexpr (V == 4) store4<T>(hr + i, (const float (&)[4]) hn); else hr[i] = from_f<T>(hn[0]);
@@ -164,24 +203,30 @@ static bool rows_by_four(const void* p, int64_t ld, int dtype)
     return p == nullptr || ((uintptr_t) p % 16 == 0 && ld % (dtype == EXL3_MIX_BF16 ? 8 : 4) == 0);
 }
 
+extern "C" int exl3_mix_residual_norm_conv(float* x, const void* y, int64_t y_ld, const void* y2, int64_t y2_ld, float y_scale, int mode, int center, const float* w,
+                                           const float* bias, float eps, void* h, int64_t h_ld, void* hn_out, int64_t hn_ld, const float* conv_w, int taps, void* ring,
+                                           const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots, int n, int width, int dtype, void* stream)
+{
+    MIX_CHECK(x && n >= 0 && width > 0 && mode >= 0 && mode <= 2, "mix_residual_norm_conv: bad arguments");
+    MIX_CHECK(mode == 0 || (y && y_ld >= width && (!y2 || y2_ld >= width)), "mix_residual_norm_conv: an addend is needed");
+    MIX_CHECK((!h && !hn_out) || (w && (!h || h_ld >= width) && (!hn_out || hn_ld >= width)), "mix_residual_norm_conv: the norm needs its weight");
+    MIX_CHECK(center || !bias, "mix_residual_norm_conv: a bias goes with the layer norm");
+    MIX_CHECK(!conv_w || (h && ring && tok_seq && tok_pos && slots && taps >= 1 && taps <= CN_MAX_TAPS), "mix_residual_norm_conv: the convolution needs 1..%d taps, the ring and the step's rows", CN_MAX_TAPS);
+    if (n == 0 || (mode == 0 && !h && !hn_out)) return EXL3_MIX_OK;
+    const bool by4 = width % 8 == 0 && (uintptr_t) x % 16 == 0 && rows_by_four(y, y_ld, dtype) && rows_by_four(y2, y2_ld, dtype) && rows_by_four(h, h_ld, dtype) &&
+                     rows_by_four(hn_out, hn_ld, dtype) && rows_by_four(ring, 8, dtype) && (uintptr_t) w % 16 == 0 && (uintptr_t) conv_w % 16 == 0;
+    #define RN_LAUNCH(VV, CC) hipLaunchKernelGGL((residual_rms_kernel<T, VV, CC>), dim3(n), dim3(CN_THREADS), 0, (hipStream_t) stream, x, (const T*) y, y_ld, (const T*) y2, y2_ld, y_scale, \
+                                                 mode, w, bias, eps, (T*) h, h_ld, (T*) hn_out, hn_ld, conv_w, taps, (T*) ring, tok_seq, tok_pos, slots, width)
+    MIX_DISPATCH_T(dtype, if (by4) { if (center) RN_LAUNCH(4, true); else RN_LAUNCH(4, false); } else { if (center) RN_LAUNCH(1, true); else RN_LAUNCH(1, false); });
+    #undef RN_LAUNCH
+    return mix_check_launch("mix_residual_norm_conv");
+}
+
 extern "C" int exl3_mix_residual_rms(float* x, const void* y, int64_t y_ld, int mode, const float* w, float eps, void* h, int64_t h_ld,
                                      const float* conv_w, int taps, void* ring, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots,
                                      int n, int width, int dtype, void* stream)
 {
-    MIX_CHECK(x && n >= 0 && width > 0 && mode >= 0 && mode <= 2, "mix_residual_rms: bad arguments");
-    MIX_CHECK(mode == 0 || (y && y_ld >= width), "mix_residual_rms: an addend is needed");
-    MIX_CHECK(!h || (w && h_ld >= width), "mix_residual_rms: the norm needs its weight");
-    MIX_CHECK(!conv_w || (h && ring && tok_seq && tok_pos && slots && taps >= 1 && taps <= CN_MAX_TAPS), "mix_residual_rms: the convolution needs 1..%d taps, the ring and the step's rows", CN_MAX_TAPS);
-    if (n == 0 || (mode == 0 && !h)) return EXL3_MIX_OK;
-    const bool by4 = width % 8 == 0 && (uintptr_t) x % 16 == 0 && rows_by_four(y, y_ld, dtype) && rows_by_four(h, h_ld, dtype) && rows_by_four(ring, 8, dtype) &&
-                     (uintptr_t) w % 16 == 0 && (uintptr_t) conv_w % 16 == 0;
-    if (by4)
-        MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((residual_rms_kernel<T, 4>), dim3(n), dim3(CN_THREADS), 0, (hipStream_t) stream, x, (const T*) y, y_ld, mode, w, eps, (T*) h, h_ld,
-                                                 conv_w, taps, (T*) ring, tok_seq, tok_pos, slots, width));
-    else
-        MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((residual_rms_kernel<T, 1>), dim3(n), dim3(CN_THREADS), 0, (hipStream_t) stream, x, (const T*) y, y_ld, mode, w, eps, (T*) h, h_ld,
-                                                 conv_w, taps, (T*) ring, tok_seq, tok_pos, slots, width));
-    return mix_check_launch("mix_residual_rms");
+    return exl3_mix_residual_norm_conv(x, y, y_ld, nullptr, 0, 1.0f, mode, 0, w, nullptr, eps, h, h_ld, nullptr, 0, conv_w, taps, ring, tok_seq, tok_pos, slots, n, width, dtype, stream);
 }
 
 extern "C" int exl3_mix_canon(void* out, int64_t out_ld, const void* hn, int64_t hn_ld, const float* conv_w, int taps, void* ring,

@@ -34,6 +34,19 @@ __device__ __forceinline__ float wave_max(float v)
     return v;
 }
 
+// sum over each row of 16 consecutive lanes, every lane of the row gets it: two quad permutes, then the mirror within 8 and within 16 lanes (data-parallel
+// primitives of the vector unit: no trip through the LDS crossbar)
+__device__ __forceinline__ float row16_sum(float v)
+{
+    #define MIX_DPP(x, ctrl) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), ctrl, 0xf, 0xf, true))
+    v += MIX_DPP(v, 0xB1);
+    v += MIX_DPP(v, 0x4E);
+    v += MIX_DPP(v, 0x141);
+    v += MIX_DPP(v, 0x140);
+    #undef MIX_DPP
+    return v;
+}
+
 // sum over a workgroup of NW waves; every thread gets the result.  `red` holds NW floats; two barriers.
 template <int NW>
 __device__ __forceinline__ float block_sum(float v, float* red)
@@ -70,6 +83,8 @@ __device__ __forceinline__ float act_f(float v, int kind)
 }
 // log(sigmoid(z)) without cancellation on either side
 __device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+// log(1 + exp(z)) without overflow
+__device__ __forceinline__ float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 
 // error reporting shared by the translation units of this library (thread-local message, negative return codes)
 void mix_set_error(const char* fmt, ...);

@@ -24,6 +24,43 @@ __global__ __launch_bounds__(ROW_THREADS) void embed_copy_kernel(float* __restri
     }
 }
 
+// x[n] = table[tokens[n]] * scale + P(tok_pos[n]): a sinusoidal position vector, entry 2i = sin(p f_i), entry 2i + 1 = cos(p f_i), f_i = freq[i] (float32;
+// the angle is the float32 product of the position and the frequency)
+template <typename T>
+__global__ __launch_bounds__(ROW_THREADS) void embed_sinusoid_kernel(float* __restrict__ x, const T* __restrict__ table, const int32_t* __restrict__ tokens,
+                                                                     const int32_t* __restrict__ tok_pos, const float* __restrict__ freq, float scale, int width, int vocab)
+{
+    const int n = blockIdx.x;
+    int tok = tokens[n];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    const T* src = table + (int64_t) tok * width;
+    const float p = (float) tok_pos[n];
+    for (int i = threadIdx.x; i < width; i += ROW_THREADS)
+    {
+        const float a = p * freq[i >> 1];
+        x[(int64_t) n * width + i] = to_f(src[i]) * scale + ((i & 1) ? cosf(a) : sinf(a));
+    }
+}
+
+// h[i] = layer norm of residual row rows[i] (or i): (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b
+template <typename T>
+__global__ __launch_bounds__(ROW_THREADS) void layer_norm_rows_kernel(T* __restrict__ h, const float* __restrict__ x, const int32_t* __restrict__ rows,
+                                                                      const float* __restrict__ w, const float* __restrict__ b, float eps, int width)
+{
+    __shared__ float red[ROW_WAVES];
+    const int n = blockIdx.x;
+    const float* xr = x + (int64_t) (rows ? rows[n] : n) * width;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < width; i += ROW_THREADS) s += xr[i];
+    const float mean = block_sum<ROW_WAVES>(s, red) / (float) width;
+    float dd = 0.f;
+    for (int i = threadIdx.x; i < width; i += ROW_THREADS) { const float d = xr[i] - mean; dd += d * d; }
+    dd = block_sum<ROW_WAVES>(dd, red);
+    const float inv = 1.0f / sqrtf(dd / (float) width + eps);
+    T* hr = h + (int64_t) n * width;
+    for (int i = threadIdx.x; i < width; i += ROW_THREADS) hr[i] = from_f<T>((xr[i] - mean) * inv * w[i] + (b ? b[i] : 0.f));
+}
+
 // mode 0: x stays; 1: x += y'; 2: x = y'   with y' = y, or y / rms(y) * rms_w when rms_w is given.
 // out 0: nothing; 1: h = x in the activation type; 2: h = tanh(alpha x) w + b.
 template <typename T>
@@ -91,23 +128,30 @@ __global__ __launch_bounds__(256) void act_kernel(T* __restrict__ out, const T* 
     else out[(int64_t) n * ff + i] = from_f<T>(act_f(to_f(z[(int64_t) n * z_ld + i]), kind));
 }
 
+// rg (optional): one number per row; the row's result is multiplied by sigmoid(rg[n]) (a gate on the whole sublayer, applied before its linear down projection)
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void glu_act_kernel(T* __restrict__ out, const T* __restrict__ g, int64_t g_ld, const T* __restrict__ u, int64_t u_ld, int ff, int kind, float limit)
+__global__ __launch_bounds__(256) void glu_act_kernel(T* __restrict__ out, const T* __restrict__ g, int64_t g_ld, const T* __restrict__ u, int64_t u_ld, int ff, int kind, float limit,
+                                                      const T* __restrict__ rg, int64_t rg_ld)
 {
     constexpr int VN = VEC ? rvec<T>::N : 1;
     const int n = blockIdx.y;
     const int i = (blockIdx.x * 256 + threadIdx.x) * VN;
     if (i >= ff) return;
+    const float rs = rg ? sigmoid_f(to_f(rg[(int64_t) n * rg_ld])) : 1.0f;
     if (VEC)
     {
         union { uint4 v; T e[rvec<T>::N]; } a, b, o;
         a.v = *(const uint4*) (g + (int64_t) n * g_ld + i);
         b.v = *(const uint4*) (u + (int64_t) n * u_ld + i);
         #pragma unroll
-        for (int e = 0; e < rvec<T>::N; ++e) o.e[e] = from_f<T>(glu_act_f(to_f(a.e[e]), to_f(b.e[e]), kind, limit));
+        for (int e = 0; e < rvec<T>::N; ++e) { const float r = glu_act_f(to_f(a.e[e]), to_f(b.e[e]), kind, limit); o.e[e] = from_f<T>(rg ? r * rs : r); }
         *(uint4*) (out + (int64_t) n * ff + i) = o.v;
     }
-    else out[(int64_t) n * ff + i] = from_f<T>(glu_act_f(to_f(g[(int64_t) n * g_ld + i]), to_f(u[(int64_t) n * u_ld + i]), kind, limit));
+    else
+    {
+        const float r = glu_act_f(to_f(g[(int64_t) n * g_ld + i]), to_f(u[(int64_t) n * u_ld + i]), kind, limit);
+        out[(int64_t) n * ff + i] = from_f<T>(rg ? r * rs : r);
+    }
 }
 
 // out[n][j] = gelu_tanh(gate[n][j]) * table[tokens[n]][col0 + j]
@@ -176,7 +220,7 @@ __global__ void topk_sigmoid_kernel(int32_t* __restrict__ idx, float* __restrict
 #define TG_MAX_PER_LANE 8
 __global__ __launch_bounds__(64) void topk_grouped_kernel(int32_t* __restrict__ idx, float* __restrict__ wts, float* __restrict__ idw, const float* __restrict__ logits,
                                                           const float* __restrict__ correction, int kind, float scale, int normalise, int groups, int keep,
-                                                          int total, int real, int top)
+                                                          int total, int real, int top, int group_top)
 {
     __shared__ float gmax[64];
     const int n = blockIdx.x, lane = threadIdx.x;
@@ -214,13 +258,30 @@ __global__ __launch_bounds__(64) void topk_grouped_kernel(int32_t* __restrict__ 
     if (groups > 1 && keep < groups)
     {
         const int per = total / groups;
-        for (int g = 0; g < groups; ++g)
+        for (int g = 0; g < groups; ++g)                     // a group's score: the sum of its `group_top` largest choice scores (1: its largest)
         {
-            float m = -INFINITY;
-            #pragma unroll
-            for (int i = 0; i < TG_MAX_PER_LANE; ++i) { const int e = lane + 64 * i; if (e < total && e / per == g) m = fmaxf(m, c[i]); }
-            m = wave_max(m);
-            if (lane == 0) gmax[g] = m;
+            unsigned used = 0u;
+            float total_g = 0.f;
+            for (int t = 0; t < group_top && t < per; ++t)
+            {
+                float bv = -INFINITY; int be = 0x7fffffff;
+                #pragma unroll
+                for (int i = 0; i < TG_MAX_PER_LANE; ++i)
+                {
+                    const int e = lane + 64 * i;
+                    if (e < total && e / per == g && !((used >> i) & 1u) && (c[i] > bv || be == 0x7fffffff)) { bv = c[i]; be = e; }
+                }
+                #pragma unroll
+                for (int o = 32; o > 0; o >>= 1)
+                {
+                    const float ov = __shfl_xor(bv, o, 64); const int oe = __shfl_xor(be, o, 64);
+                    if (oe != 0x7fffffff && (be == 0x7fffffff || ov > bv || (ov == bv && oe < be))) { bv = ov; be = oe; }
+                }
+                #pragma unroll
+                for (int i = 0; i < TG_MAX_PER_LANE; ++i) if (lane + 64 * i == be) used |= 1u << i;
+                total_g = t == 0 ? bv : total_g + bv;
+            }
+            if (lane == 0) gmax[g] = total_g;
         }
         __syncthreads();
         unsigned long long kept = 0ull;                      // every lane picks the same groups: the `keep` largest, ties to the lower index
@@ -280,6 +341,23 @@ __global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, int
     for (int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t) gridDim.x * 256) x[i] = cap * tanhf(x[i] / cap);
 }
 
+extern "C" int exl3_mix_embed_sinusoid(float* x, const void* table, const int32_t* tokens, const int32_t* tok_pos, const float* freq, float scale, int n, int width, int vocab,
+                                       int dtype, void* stream)
+{
+    MIX_CHECK(x && table && tokens && tok_pos && freq && n >= 0 && width > 0 && vocab > 0, "mix_embed_sinusoid: bad arguments");
+    if (n == 0) return EXL3_MIX_OK;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(embed_sinusoid_kernel<T>, dim3(n), dim3(ROW_THREADS), 0, (hipStream_t) stream, x, (const T*) table, tokens, tok_pos, freq, scale, width, vocab));
+    return mix_check_launch("mix_embed_sinusoid");
+}
+
+extern "C" int exl3_mix_layer_norm_rows(void* h, const float* x, const int32_t* rows, const float* w, const float* b, float eps, int n, int width, int dtype, void* stream)
+{
+    MIX_CHECK(h && x && w && n >= 0 && width > 0, "mix_layer_norm_rows: bad arguments");
+    if (n == 0) return EXL3_MIX_OK;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(layer_norm_rows_kernel<T>, dim3(n), dim3(ROW_THREADS), 0, (hipStream_t) stream, (T*) h, x, rows, w, b, eps, width));
+    return mix_check_launch("mix_layer_norm_rows");
+}
+
 extern "C" int exl3_mix_embed_copy(float* x, void* xc, int64_t xc_ld, const void* table, const int32_t* tokens, int n, int width, int vocab, int dtype, void* stream)
 {
     MIX_CHECK(x && table && tokens && n >= 0 && width > 0 && vocab > 0 && (!xc || xc_ld >= width), "mix_embed_copy: bad arguments");
@@ -329,7 +407,13 @@ extern "C" int exl3_mix_act(void* out, const void* z, int64_t z_ld, int n, int f
 
 extern "C" int exl3_mix_glu_act(void* out, const void* g, int64_t g_ld, const void* u, int64_t u_ld, int n, int ff, int kind, float limit, int dtype, void* stream)
 {
-    MIX_CHECK(out && g && u && n >= 0 && ff > 0 && g_ld >= ff && u_ld >= ff && kind >= 0 && kind <= 1, "mix_glu_act: bad arguments");
+    return exl3_mix_glu_act_rowgate(out, g, g_ld, u, u_ld, nullptr, 0, n, ff, kind, limit, dtype, stream);
+}
+
+extern "C" int exl3_mix_glu_act_rowgate(void* out, const void* g, int64_t g_ld, const void* u, int64_t u_ld, const void* rg, int64_t rg_ld, int n, int ff, int kind, float limit,
+                                        int dtype, void* stream)
+{
+    MIX_CHECK(out && g && u && n >= 0 && ff > 0 && g_ld >= ff && u_ld >= ff && kind >= 0 && kind <= 1 && (!rg || rg_ld >= 1), "mix_glu_act: bad arguments");
     const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
     const bool vec = ff % vn == 0 && g_ld % vn == 0 && u_ld % vn == 0 && (uintptr_t) out % 16 == 0 && (uintptr_t) g % 16 == 0 && (uintptr_t) u % 16 == 0;
     for (int r0 = 0; r0 < n; r0 += 65535)
@@ -337,10 +421,12 @@ extern "C" int exl3_mix_glu_act(void* out, const void* g, int64_t g_ld, const vo
         const int rows = n - r0 < 65535 ? n - r0 : 65535;
         if (vec)
             MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((glu_act_kernel<T, true>), dim3((ff / vn + 255) / 256, rows), dim3(256), 0, (hipStream_t) stream, (T*) out + (int64_t) r0 * ff,
-                                                     (const T*) g + (int64_t) r0 * g_ld, g_ld, (const T*) u + (int64_t) r0 * u_ld, u_ld, ff, kind, limit));
+                                                     (const T*) g + (int64_t) r0 * g_ld, g_ld, (const T*) u + (int64_t) r0 * u_ld, u_ld, ff, kind, limit,
+                                                     rg ? (const T*) rg + (int64_t) r0 * rg_ld : nullptr, rg_ld));
         else
             MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((glu_act_kernel<T, false>), dim3((ff + 255) / 256, rows), dim3(256), 0, (hipStream_t) stream, (T*) out + (int64_t) r0 * ff,
-                                                     (const T*) g + (int64_t) r0 * g_ld, g_ld, (const T*) u + (int64_t) r0 * u_ld, u_ld, ff, kind, limit));
+                                                     (const T*) g + (int64_t) r0 * g_ld, g_ld, (const T*) u + (int64_t) r0 * u_ld, u_ld, ff, kind, limit,
+                                                     rg ? (const T*) rg + (int64_t) r0 * rg_ld : nullptr, rg_ld));
     }
     return mix_check_launch("mix_glu_act");
 }
@@ -375,12 +461,19 @@ extern "C" int exl3_mix_topk_sigmoid(int32_t* idx, float* wts, const float* logi
 extern "C" int exl3_mix_topk_grouped(int32_t* idx, float* wts, float* idw, const float* logits, const float* correction, int kind, float scale, int normalise,
                                      int groups, int keep, int n, int total, int real, int top, void* stream)
 {
+    return exl3_mix_topk_grouped_ex(idx, wts, idw, logits, correction, kind, scale, normalise, groups, keep, 1, n, total, real, top, stream);
+}
+
+extern "C" int exl3_mix_topk_grouped_ex(int32_t* idx, float* wts, float* idw, const float* logits, const float* correction, int kind, float scale, int normalise,
+                                        int groups, int keep, int group_top, int n, int total, int real, int top, void* stream)
+{
+    MIX_CHECK(group_top >= 1, "mix_topk_grouped: a group's score is the sum of at least one choice score");
     MIX_CHECK(idx && wts && logits && n >= 0 && total > 0 && real >= 0 && real <= total && (real == total || idw), "mix_topk_grouped: bad arguments");
     MIX_CHECK(total <= 64 * TG_MAX_PER_LANE && top > 0 && top <= 64 && top <= total && (kind == 0 || kind == 1), "mix_topk_grouped: at most %d outputs, top <= 64", 64 * TG_MAX_PER_LANE);
     MIX_CHECK(groups >= 1 && groups <= 64 && total % groups == 0 && keep >= 1 && keep <= groups && top <= keep * (total / groups),
               "mix_topk_grouped: %d groups (keep %d) over %d outputs cannot give %d choices", groups, keep, total, top);
     if (n == 0) return EXL3_MIX_OK;
-    hipLaunchKernelGGL(topk_grouped_kernel, dim3(n), dim3(64), 0, (hipStream_t) stream, idx, wts, idw, logits, correction, kind, scale, normalise, groups, keep, total, real, top);
+    hipLaunchKernelGGL(topk_grouped_kernel, dim3(n), dim3(64), 0, (hipStream_t) stream, idx, wts, idw, logits, correction, kind, scale, normalise, groups, keep, total, real, top, group_top);
     return mix_check_launch("mix_topk_grouped");
 }
 

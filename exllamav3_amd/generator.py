@@ -85,6 +85,7 @@ class Generator:
         """One token per sequence: eager the first time a batch size occurs, captured the second time, replayed afterwards."""
         if not self.graphs:
             return self.model.step(self.cache.begin_step(entries), self.cache)
+        self.cache.reserve(entries)                # a cache with pages may grow here: before the graphs' addresses are trusted
         if self._generation != self.cache.generation:
             self._graphs.clear(); self._seen.clear()
             self._generation = self.cache.generation

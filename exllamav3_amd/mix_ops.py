@@ -632,3 +632,204 @@ def moe_grouped_plain(y, h, wu, wd, idx, wts, act_kind: int, idw=None):
         at += c
     _check(lib.exl3_mix_moe_combine_id(_p(y), _p(out), _p(where), _p(wts), _p(idx), experts, _p(h) if idw is not None else None, _p(idw), n, top, width,
                                         code(h.dtype), _stream(h)))
+
+
+# ---- parallel blocks over a layer norm, attention without softmax over paged keys, recurrent mixers with a scalar decay per head ----
+
+GATE_SILU, GATE_SIGMOID = 0, 1
+SIG_MFMA_MIN_ROWS = 32
+
+
+def embed_sinusoid(x: torch.Tensor, table: torch.Tensor, tokens: torch.Tensor, tok_pos: torch.Tensor, freq: torch.Tensor, scale: float):
+    """x (float32) = table[tokens] * scale + the sinusoidal vector of each row's position (freq: float32 [ceil(width / 2)])."""
+    n, width = x.shape
+    _f32c(x, "x"); _f32c(freq, "freq"); _i32c(tokens, "tokens"); _i32c(tok_pos, "tok_pos")
+    _req(tokens.numel() == n and tok_pos.numel() == n and table.is_contiguous() and table.shape[1] == width and freq.numel() >= (width + 1) // 2, "embed_sinusoid: shapes")
+    _check(_lib.mixlib().exl3_mix_embed_sinusoid(_p(x), _p(table), _p(tokens), _p(tok_pos), _p(freq), scale, n, width, table.shape[0], code(table.dtype), _stream(x)))
+
+
+def layer_norm_rows(h: torch.Tensor, x: torch.Tensor, rows: torch.Tensor | None, w: torch.Tensor, b: torch.Tensor | None, eps: float):
+    n, width = h.shape
+    _f32c(x, "x"); _f32c(w, "w")
+    _req(h.is_contiguous() and x.shape[1] == width and w.numel() == width, "layer_norm_rows: shapes")
+    if b is not None:
+        _f32c(b, "b"); _req(b.numel() == width, "layer_norm_rows: bias")
+    if rows is not None:
+        _i32c(rows, "rows"); _req(rows.numel() == n, "layer_norm_rows: rows")
+    else:
+        _req(x.shape[0] == n, "layer_norm_rows: rows of x")
+    _check(_lib.mixlib().exl3_mix_layer_norm_rows(_p(h), _p(x), _p(rows), _p(w), _p(b), eps, n, width, code(h.dtype), _stream(x)))
+
+
+def residual_norm_conv(x, y_view, y2_view, y_scale: float, mode: int, center: bool, w, bias, eps: float, h_view, hn_view=None, conv_w=None, ring=None, tok_seq=None,
+                       tok_pos=None, slots=None):
+    """x (float32, in place) = x | x + (y + y2) * y_scale | (y + y2) * y_scale; then the norm of x (center: layer norm with weight and optional bias, else RMS norm
+    with weight) into hn_view and / or h_view; with conv_w [taps, width] (steps of one row per sequence) h = normed row + its causal convolution over the slot's
+    ring, which receives the new normed row."""
+    n, width = x.shape
+    _f32c(x, "x")
+    ref = next((t for t in (y_view, h_view, hn_view) if t is not None), None)
+    _req(ref is not None, "residual_norm_conv: nothing to do")
+    if mode != RES_KEEP:
+        _req(y_view is not None and y_view.shape[0] == n and (y2_view is None or (y2_view.shape[0] == n and y2_view.dtype == y_view.dtype)), "residual_norm_conv: y")
+    else:
+        y_view = y2_view = None
+    if h_view is not None or hn_view is not None:
+        _f32c(w, "w"); _req(w.numel() == width, "residual_norm_conv: w")
+        if bias is not None:
+            _f32c(bias, "bias"); _req(bias.numel() == width and center, "residual_norm_conv: bias")
+        for t in (h_view, hn_view):
+            _req(t is None or (t.shape[0] == n and t.dtype == ref.dtype), "residual_norm_conv: h")
+    taps = 0
+    if conv_w is not None:
+        _f32c(conv_w, "conv_w"); taps = conv_w.shape[0]
+        _req(conv_w.shape[1] == width and ring is not None and ring.is_contiguous() and ring.shape[1:] == (max(taps - 1, 1), width) and ring.dtype == ref.dtype,
+             "residual_norm_conv: convolution weights / ring")
+        for t, nm in ((tok_seq, "tok_seq"), (tok_pos, "tok_pos"), (slots, "slots")):
+            _i32c(t, nm)
+    ld = lambda t, nm: 0 if t is None else _view(t, width, nm)
+    _check(_lib.mixlib().exl3_mix_residual_norm_conv(_p(x), _p(y_view), ld(y_view, "y"), _p(y2_view), ld(y2_view, "y2"), y_scale, mode, 1 if center else 0, _p(w), _p(bias), eps,
+                                                      _p(h_view), ld(h_view, "h"), _p(hn_view), ld(hn_view, "hn"), _p(conv_w), taps, _p(ring), _p(tok_seq), _p(tok_pos), _p(slots),
+                                                      n, width, code(ref.dtype), _stream(x)))
+
+
+def glu_act_rowgate(out: torch.Tensor, g_view: torch.Tensor, u_view: torch.Tensor, row_gate: torch.Tensor | None, kind: int, limit: float = 0.0):
+    """out = glu(g, u) * sigmoid(row_gate[n]) (row_gate: [n, 1] view, one number per row)."""
+    n, ff = out.shape
+    _req(out.is_contiguous() and g_view.dtype == out.dtype == u_view.dtype and g_view.shape[0] == n and u_view.shape[0] == n, "glu_act_rowgate: shapes")
+    if row_gate is not None:
+        _req(row_gate.dtype == out.dtype and row_gate.shape == (n, 1), "glu_act_rowgate: the gate is one number per row")
+    _check(_lib.mixlib().exl3_mix_glu_act_rowgate(_p(out), _p(g_view), _view(g_view, ff, "g"), _p(u_view), _view(u_view, ff, "u"), _p(row_gate),
+                                                   0 if row_gate is None else max(row_gate.stride(0), 1), n, ff, kind, limit, code(out.dtype), _stream(out)))
+
+
+def topk_grouped_ex(idx, wts, idw, logits, correction, kind: int, real: int, groups: int = 1, keep: int = 1, group_top: int = 1, scale: float = 1.0, normalise: bool = True):
+    """topk_grouped with a group's score = the sum of its `group_top` largest choice scores."""
+    n, total = logits.shape
+    top = idx.shape[1]
+    _f32c(logits, "logits"); _f32c(wts, "wts"); _i32c(idx, "idx")
+    _req(idx.shape == wts.shape == (n, top), "topk_grouped: shapes")
+    if idw is not None:
+        _f32c(idw, "idw"); _req(idw.numel() == n, "topk_grouped: idw")
+    if correction is not None:
+        _f32c(correction, "correction"); _req(correction.numel() == total, "topk_grouped: correction")
+    _check(_lib.mixlib().exl3_mix_topk_grouped_ex(_p(idx), _p(wts), _p(idw), _p(logits), _p(correction), kind, scale, 1 if normalise else 0, groups, keep, group_top, n, total, real,
+                                                   top, _stream(logits)))
+
+
+def _paged(k_pages, v_pages, table, name):
+    _i32c(table, "page table")
+    _req(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.dim() == 3 and v_pages.dim() == 3 and k_pages.shape[:2] == v_pages.shape[:2] and table.dim() == 2
+         and k_pages.dtype == v_pages.dtype, f"{name}: pools [pages, page, width] and a table [slots, pages per slot]")
+
+
+def paged_store(k_pages, v_pages, k_view, v_view, table, tok_seq, tok_pos, slots):
+    """The step's key / value rows into the pages of their sequences (pools [pages, page, kw] / [pages, page, vw])."""
+    _paged(k_pages, v_pages, table, "paged_store")
+    n = k_view.shape[0]
+    kw, vw = k_pages.shape[2], v_pages.shape[2]
+    for t, nm in ((tok_seq, "tok_seq"), (tok_pos, "tok_pos"), (slots, "slots")):
+        _i32c(t, nm)
+    _req(k_view.dtype == k_pages.dtype == v_view.dtype and v_view.shape[0] == n and tok_seq.numel() == n, "paged_store: rows")
+    _check(_lib.mixlib().exl3_mix_paged_store(_p(k_pages), _p(v_pages), _p(k_view), _view(k_view, kw, "k"), _p(v_view), _view(v_view, vw, "v"), _p(table), table.stride(0),
+                                               k_pages.shape[1], _p(tok_seq), _p(tok_pos), _p(slots), n, kw, vw, code(k_view.dtype), _stream(k_view)))
+
+
+def sig_mfma_ok(dtype, max_rows: int, dim: int, vdim: int) -> bool:
+    return dtype == torch.bfloat16 and max_rows >= SIG_MFMA_MIN_ROWS and dim <= 256 and vdim <= 256
+
+
+def sigattn_prefill(out, q_view, k_view, v_view, bias, cu, tok_seq, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, max_rows: int):
+    """Prompt steps of the attention without softmax: out [n, heads * vdim] = sum over the row's keys of sigmoid(scale q.k + bias[head]) v.  bfloat16 steps of at
+    least SIG_MFMA_MIN_ROWS rows run on the matrix cores, everything else in the exact float32-score kernel."""
+    n = out.shape[0]
+    _i32c(cu, "cu"); _i32c(tok_seq, "tok_seq")
+    if bias is not None:
+        _f32c(bias, "bias"); _req(bias.numel() == heads, "sigattn_prefill: one bias per head")
+    _req(out.is_contiguous() and out.shape == (n, heads * vdim) and q_view.dtype == out.dtype == k_view.dtype == v_view.dtype, "sigattn_prefill: shapes")
+    args = (_p(out), _p(q_view), _view(q_view, heads * dim, "q"), _p(k_view), _view(k_view, kv_heads * dim, "k"), _p(v_view), _view(v_view, kv_heads * vdim, "v"), _p(bias), _p(cu))
+    if sig_mfma_ok(out.dtype, max_rows, dim, vdim):
+        _check(_lib.mixlib().exl3_mix_sigattn_prefill_mfma(*args, cu.numel() - 1, max_rows, heads, kv_heads, dim, vdim, scale, _stream(out)))
+    else:
+        _check(_lib.mixlib().exl3_mix_sigattn_prefill(*args, _p(tok_seq), n, heads, kv_heads, dim, vdim, scale, code(out.dtype), _stream(out)))
+
+
+def sigattn_decode(out, q_view, k_pages, v_pages, bias, table, slots, len_after, heads: int, kv_heads: int, dim: int, vdim: int, scale: float):
+    """Decode steps (one row per sequence): every sequence reads its len_after keys through the page table."""
+    _paged(k_pages, v_pages, table, "sigattn_decode")
+    n = out.shape[0]
+    _i32c(slots, "slots"); _i32c(len_after, "len_after")
+    if bias is not None:
+        _f32c(bias, "bias"); _req(bias.numel() == heads, "sigattn_decode: one bias per head")
+    _req(out.is_contiguous() and out.shape == (n, heads * vdim) and q_view.dtype == out.dtype == k_pages.dtype and k_pages.shape[2] == kv_heads * dim
+         and v_pages.shape[2] == kv_heads * vdim and slots.numel() == n, "sigattn_decode: shapes")
+    _check(_lib.mixlib().exl3_mix_sigattn_decode(_p(out), _p(q_view), _view(q_view, heads * dim, "q"), _p(k_pages), _p(v_pages), _p(bias), _p(table), table.stride(0),
+                                                  k_pages.shape[1], _p(slots), _p(len_after), n, heads, kv_heads, dim, vdim, scale, code(out.dtype), _stream(out)))
+
+
+def mlstm_scan(o, S, nst, mst, q_view, k_view, v_view, zi_view, zf_view, bias_i, bias_f, cu, slots, pos0, q_scale: float, cap: float):
+    """o [n, heads, vdim] float32; state per slot S [heads, vdim, dim], n [heads, dim], m [heads] (float32)."""
+    n, heads, vdim = o.shape
+    dim = S.shape[3]
+    for t, nm in ((o, "o"), (S, "S"), (nst, "n"), (mst, "m"), (bias_i, "bias_i"), (bias_f, "bias_f")):
+        _f32c(t, nm)
+    for t, nm in ((cu, "cu"), (slots, "slots"), (pos0, "pos0")):
+        _i32c(t, nm)
+    _req(S.shape[1:] == (heads, vdim, dim) and nst.shape[1:] == (heads, dim) and mst.shape[1:] == (heads,) and bias_i.numel() == heads and bias_f.numel() == heads
+         and q_view.dtype == k_view.dtype == v_view.dtype == zi_view.dtype == zf_view.dtype, "mlstm_scan: shapes")
+    _check(_lib.mixlib().exl3_mix_mlstm_scan(_p(o), _p(S), _p(nst), _p(mst), _p(q_view), _view(q_view, heads * dim, "q"), _p(k_view), _view(k_view, heads * dim, "k"),
+                                              _p(v_view), _view(v_view, heads * vdim, "v"), _p(zi_view), _view(zi_view, heads, "zi"), _p(zf_view), _view(zf_view, heads, "zf"),
+                                              _p(bias_i), _p(bias_f), _p(cu), _p(slots), _p(pos0), cu.numel() - 1, heads, dim, vdim, q_scale, cap, code(q_view.dtype), _stream(o)))
+
+
+def delta_prep(qo, ko, vo, beta, decay, x_view, conv_w, ring, zb_view, za_view, A_log, dt_bias, tok_seq, tok_pos, slots, pos0, len_after, heads: int, kv_heads: int, dim: int,
+               vdim: int, q_scale: float):
+    """The delta rule's input stage over x = q | k | v [n, C]: short convolutions (conv_w [taps, C], ring [slots, taps - 1, C]) with silu, unit query / key vectors,
+    beta and decay; float32 results."""
+    n = x_view.shape[0]
+    C = 2 * kv_heads * dim + heads * vdim
+    taps = conv_w.shape[0]
+    for t, nm in ((qo, "qo"), (ko, "ko"), (vo, "vo"), (beta, "beta"), (decay, "decay"), (conv_w, "conv_w"), (A_log, "A_log"), (dt_bias, "dt_bias")):
+        _f32c(t, nm)
+    for t, nm in ((tok_seq, "tok_seq"), (tok_pos, "tok_pos"), (slots, "slots"), (pos0, "pos0"), (len_after, "len_after")):
+        _i32c(t, nm)
+    _req(qo.shape == ko.shape == (n, kv_heads * dim) and vo.shape == (n, heads * vdim) and beta.shape == decay.shape == (n, heads) and conv_w.shape[1] == C
+         and ring.is_contiguous() and ring.shape[1:] == (max(taps - 1, 1), C) and ring.dtype == x_view.dtype == zb_view.dtype == za_view.dtype
+         and A_log.numel() == heads and dt_bias.numel() == heads, "delta_prep: shapes")
+    _check(_lib.mixlib().exl3_mix_delta_prep(_p(qo), _p(ko), _p(vo), _p(beta), _p(decay), _p(x_view), _view(x_view, C, "x"), _p(conv_w), taps, _p(ring),
+                                              _p(zb_view), _view(zb_view, heads, "zb"), _p(za_view), _view(za_view, heads, "za"), _p(A_log), _p(dt_bias),
+                                              _p(tok_seq), _p(tok_pos), _p(slots), _p(pos0), _p(len_after), n, heads, kv_heads, dim, vdim, q_scale, code(x_view.dtype), _stream(qo)))
+
+
+def delta_scan(o, S, q, k, v, beta, decay, cu, slots, pos0, kv_heads: int):
+    """o [n, heads, vdim] float32; state per slot S [heads, vdim, dim] float32; q / k [n, kv_heads * dim], v [n, heads * vdim], beta / decay [n, heads] float32."""
+    n, heads, vdim = o.shape
+    dim = S.shape[3]
+    for t, nm in ((o, "o"), (S, "S"), (q, "q"), (k, "k"), (v, "v"), (beta, "beta"), (decay, "decay")):
+        _f32c(t, nm)
+    for t, nm in ((cu, "cu"), (slots, "slots"), (pos0, "pos0")):
+        _i32c(t, nm)
+    _req(S.shape[1:] == (heads, vdim, dim) and q.shape == k.shape == (n, kv_heads * dim) and v.shape == (n, heads * vdim) and beta.shape == decay.shape == (n, heads),
+         "delta_scan: shapes")
+    _check(_lib.mixlib().exl3_mix_delta_scan(_p(o), _p(S), _p(q), _p(k), _p(v), _p(beta), _p(decay), _p(cu), _p(slots), _p(pos0), cu.numel() - 1, heads, kv_heads, dim, vdim,
+                                              _stream(o)))
+
+
+def head_norm_gate(out, o, w, g_view, gate: int, eps: float):
+    """out [n, heads * vdim] = o / rms(o per head) * w * gate(g); w has vdim entries (shared by the heads) or heads * vdim; gate GATE_SILU / GATE_SIGMOID."""
+    n, heads, vdim = o.shape
+    _f32c(o, "o"); _f32c(w, "w")
+    _req(out.is_contiguous() and out.shape == (n, heads * vdim) and w.numel() in (vdim, heads * vdim) and g_view.dtype == out.dtype, "head_norm_gate: shapes")
+    per_head = 1 if (w.numel() == heads * vdim and heads > 1) else 0
+    _check(_lib.mixlib().exl3_mix_head_norm_gate(_p(out), _p(o), _p(w), per_head, _p(g_view), _view(g_view, heads * vdim, "g"), gate, eps, n, heads, vdim, code(out.dtype),
+                                                  _stream(out)))
+
+
+def rms_pair(out, a_view, wa, b_view, wb, scale: float, eps: float):
+    """out = scale * (a / rms(a) * wa + b / rms(b) * wb) row by row."""
+    n, width = out.shape
+    _f32c(wa, "wa"); _f32c(wb, "wb")
+    _req(out.is_contiguous() and a_view.dtype == out.dtype == b_view.dtype and a_view.shape[0] == n and b_view.shape[0] == n and wa.numel() == width and wb.numel() == width,
+         "rms_pair: shapes")
+    _check(_lib.mixlib().exl3_mix_rms_pair(_p(out), _p(a_view), _view(a_view, width, "a"), _p(wa), _p(b_view), _view(b_view, width, "b"), _p(wb), scale, eps, n, width,
+                                            code(out.dtype), _stream(out)))

@@ -30,6 +30,14 @@ float32 accumulation; true float32 when the model runs in float32).
                             (or window) mask; rings of one chunk per slot
     CanonBlock              x += mixer(canon1(x)); x += ff(canon2(x)) over CanonNorm inputs
 
+    LayerNormConv           layer norm (weight and bias) followed by the same input convolution; hands out both the normed rows and the convolved rows
+    SigmoidAttention        grouped-query causal attention without softmax (weights sigmoid(scale q.k + bias_head), not normalised), no window: keys and
+                            values in the cache's pages
+    MatrixLSTM              matrix memory with exponential gating (mLSTM): capped log gates, running maximum, float32 state [heads, vdim, dim] + normaliser
+    GatedDeltaRule          delta-rule memory with a scalar decay per head and token, short convolutions with silu on q / k / v, unit query / key vectors
+    ParallelMixer           two mixers side by side over ONE fused input product, their outputs RMS-normed and averaged
+    ParallelBlock           x += m (mixer(conv(n(x))) + ff(n(x))): one norm, both sublayers read it, the residual factor m
+
 Every sum that the model's exactness rests on (norms, scores, softmax, decays, states, the residual) is float32 inside the kernels in
 both modes; the element type only decides how matrix products and their outputs are held.
 """
@@ -68,7 +76,16 @@ class FusedInput:
 
     def __call__(self, h: torch.Tensor) -> dict[str, torch.Tensor]:
         out = F.linear(h, self.weight, self.bias)
-        return {n: out[:, a: a + s] for n, (a, s) in self.offsets.items()}
+        p = {n: out[:, a: a + s] for n, (a, s) in self.offsets.items()}
+        p[self.ALL] = out                     # the whole product, for a consumer that reads several neighbouring parts as one block
+        return p
+
+    ALL = "*"
+
+    def block(self, p: dict, first: str, last: str) -> torch.Tensor:
+        """The column block from part `first` to part `last` (neighbours in the order they were given)."""
+        a, b = self.offsets[first][0], self.offsets[last][0] + self.offsets[last][1]
+        return p[self.ALL][:, a:b]
 
 
 class SlidingSinkAttention:
@@ -317,10 +334,13 @@ class ActMLP:
 class GatedMLP:
     KINDS = {"silu": mix_ops.GLU_SILU, "clamped_swish": mix_ops.GLU_CLAMPED_SWISH}
 
-    def __init__(self, width: int, ff: int, act: str = "silu", limit: float = 0.0):
-        self.width, self.ff, self.kind, self.limit = width, ff, self.KINDS[act], float(limit)
+    def __init__(self, width: int, ff: int, act: str = "silu", limit: float = 0.0, row_gate: str | None = None):
+        """row_gate: name of a [1, width] weight; the sublayer's output is multiplied by sigmoid(W_row_gate h), one number per row (applied to the hidden
+        activation, ahead of the linear down projection, so that the product's epilogue can still add it to another sum)."""
+        self.width, self.ff, self.kind, self.limit, self.row_gate = width, ff, self.KINDS[act], float(limit), row_gate
 
     def load(self, stc, prefix: str, dtype, device, extra_parts=()):
+        extra_parts = list(extra_parts) + ([("row_gate", _w(stc, prefix + self.row_gate, dtype, device).view(1, self.width), None)] if self.row_gate else [])
         self.inp = FusedInput([("gate", _w(stc, prefix + "gate", dtype, device), None), ("up", _w(stc, prefix + "up", dtype, device), None)] + list(extra_parts))
         self.w_down = _w(stc, prefix + "down", dtype, device)
         assert self.inp.offsets["up"][1] == self.ff and self.w_down.shape == (self.width, self.ff)
@@ -329,7 +349,10 @@ class GatedMLP:
     def hidden(self, h: torch.Tensor) -> tuple[torch.Tensor, dict]:
         p = self.inp(h)
         a = torch.empty((h.shape[0], self.ff), dtype=self.dtype, device=h.device)
-        mix_ops.glu_act(a, p["gate"], p["up"], self.kind, self.limit)
+        if self.row_gate:
+            mix_ops.glu_act_rowgate(a, p["gate"], p["up"], p["row_gate"], self.kind, self.limit)
+        else:
+            mix_ops.glu_act(a, p["gate"], p["up"], self.kind, self.limit)
         return a, p
 
     def forward(self, h: torch.Tensor, sb: StepBatch, add_to: torch.Tensor | None = None) -> tuple[torch.Tensor, dict]:
@@ -406,12 +429,12 @@ class SparseExperts:
 
     def __init__(self, width: int, ff: int, experts: int, top: int, router: str = "softmax", router_bias: bool = True, correction: bool = False,
                  route_scale: float = 1.0, act: str = "silu", limit: float = 0.0, shared: GatedMLP | None = None, gated: bool = True, identity: int = 0,
-                 groups: int = 1, keep_groups: int = 1):
+                 groups: int = 1, keep_groups: int = 1, group_top: int = 1):
         """router "softmax": the top logits, weights = softmax over them.  "sigmoid": scores sigmoid(z), chosen by score (+ a stored correction that the
         weights do not see), weights = chosen scores / their sum * route_scale.  "softmax_all": scores = softmax over all router outputs, chosen by score +
         correction inside the `keep_groups` best of `groups` groups of neighbouring outputs, weights = chosen scores / their sum * route_scale (the grouped
         form also serves "sigmoid" when groups > 1).  identity: the router has this many outputs beyond the stored experts; they stand for experts that return
-        their input.  gated False: experts are W_down act(W_up h) with a plain activation (ActMLP.KINDS).  shared: an expert that every row runs, added to
+        their input.  group_top: a group's score is the sum of its group_top largest choice scores (1: its largest).  gated False: experts are W_down act(W_up h) with a plain activation (ActMLP.KINDS).  shared: an expert that every row runs, added to
         the routed sum."""
         if not 0 < top <= experts + identity:
             raise RuntimeError(f"router: top {top} of {experts + identity} experts")
@@ -423,7 +446,7 @@ class SparseExperts:
             raise RuntimeError(f"router: {groups} groups (keep {keep_groups}) over {experts + identity} outputs cannot give {top} choices")
         self.width, self.ff, self.experts, self.top = width, ff, experts, top
         self.router, self.has_router_bias, self.has_correction, self.route_scale = router, router_bias, correction, float(route_scale)
-        self.gated, self.identity, self.groups, self.keep_groups = gated, int(identity), int(groups), int(keep_groups)
+        self.gated, self.identity, self.groups, self.keep_groups, self.group_top = gated, int(identity), int(groups), int(keep_groups), int(group_top)
         self.act_kind = GatedMLP.KINDS[act] if gated else ActMLP.KINDS[act]
         self.limit, self.shared = float(limit), shared
 
@@ -453,8 +476,8 @@ class SparseExperts:
             mix_ops.topk_sigmoid(idx, wts, logits, self.correction, self.route_scale)
         else:
             idw = torch.empty((sb.n,), dtype=torch.float32, device=h.device) if self.identity else None
-            mix_ops.topk_grouped(idx, wts, idw, logits, self.correction, mix_ops.ROUTE_SOFTMAX_ALL if self.router == "softmax_all" else mix_ops.ROUTE_SIGMOID,
-                                 self.experts, self.groups, self.keep_groups, self.route_scale)
+            mix_ops.topk_grouped_ex(idx, wts, idw, logits, self.correction, mix_ops.ROUTE_SOFTMAX_ALL if self.router == "softmax_all" else mix_ops.ROUTE_SIGMOID,
+                                    self.experts, self.groups, self.keep_groups, self.group_top, self.route_scale)
         y = torch.empty((sb.n, self.width), dtype=self.dtype, device=h.device)
         if not self.gated:
             if sb.n >= self.GROUPED_MIN_ROWS:
@@ -640,3 +663,232 @@ class CanonBlock:
             mix_ops.residual_rms(x, y, mix_ops.RES_ADD, None, self.eps, None)
             return None
         return nxt[0].apply(x, y, mix_ops.RES_ADD, sb, nxt[1])
+
+
+class LayerNormConv:
+    """What the sublayers of a parallel block read: hn = (x - mean) / sqrt(var + eps) * w + b (var = mean of the squared deviations), and h = hn + conv(hn),
+    conv(hn)_t = sum_j c[:, j] hn_(t - taps + 1 + j) per channel with zeros before the sequence's start.  Like CanonNorm it is never a kernel chain of its own:
+    the residual update before it writes it (one launch for steps of one row per sequence, two for prompt steps), and it hands out BOTH rows -- the
+    feed-forward reads hn, the mixer reads h.  The last taps - 1 normed rows of a sequence live in its slot."""
+
+    def __init__(self, width: int, taps: int, eps: float):
+        if taps < 1 or taps > 16:
+            raise RuntimeError(f"input convolution: {taps} taps")
+        self.width, self.taps, self.eps = width, int(taps), float(eps)
+        self.dtype = torch.bfloat16
+
+    def load(self, stc, norm_key: str, conv_key: str, dtype, device):
+        self.w, self.b = _f32(stc, norm_key, device), _f32(stc, norm_key + ".b", device)
+        self.conv = _f32(stc, conv_key, device).t().contiguous()               # stored [width, taps]; the kernels read one tap of neighbouring channels at once
+        assert self.w.numel() == self.width and self.b.numel() == self.width and self.conv.shape == (self.taps, self.width)
+        self.dtype = dtype
+        return self
+
+    def state_spec(self, name: str) -> StateSpec:
+        return StateSpec(name, (max(self.taps - 1, 1), self.width), self.dtype)
+
+    def apply(self, x: torch.Tensor, y: torch.Tensor | None, y2: torch.Tensor | None, scale: float, mode: int, sb: StepBatch, ring: torch.Tensor):
+        """x <- x | x + (y + y2) scale | (y + y2) scale; returns (hn, h) [n, width] in the activation type."""
+        hn = torch.empty((sb.n, self.width), dtype=self.dtype, device=x.device)
+        h = torch.empty_like(hn)
+        if sb.decode:
+            mix_ops.residual_norm_conv(x, y, y2, scale, mode, True, self.w, self.b, self.eps, h, hn, self.conv, ring, sb.tok_seq, sb.tok_pos, sb.slots)
+        else:
+            mix_ops.residual_norm_conv(x, y, y2, scale, mode, True, self.w, self.b, self.eps, None, hn)
+            mix_ops.canon(h, hn, self.conv, ring, sb.tok_seq, sb.tok_pos, sb.slots, sb.pos0, sb.len_after)
+        return hn, h
+
+
+class _SideMixer:
+    """Shared plumbing of the mixers below: a mixer either owns its fused input product (load / forward) or lends its parts to a ParallelMixer, which runs
+    one product for both of its mixers and calls `run` with the parts' views.  `tag` prefixes the mixer's part names and its state names."""
+    tag = ""
+
+    def load(self, stc, prefix: str, dtype, device, extra_parts=()):
+        self.inp = FusedInput(self.input_parts(stc, prefix, dtype, device) + list(extra_parts))
+        self.load_rest(stc, prefix, dtype, device)
+
+    def forward(self, h: torch.Tensor, sb: StepBatch, state: dict) -> tuple[torch.Tensor, dict]:
+        p = self.inp(h)
+        return self.run(p, self.inp, sb, state), p
+
+
+class SigmoidAttention(_SideMixer):
+    """H query heads over G key/value heads, no biases, no rotation (positions do not enter the scores), causal without a window.  The weight of a visible key
+    is sigmoid(scale q.k + bias_head); weights are NOT normalised over keys.  Keys and values of every token stay: they live in the cache's pages."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float):
+        if heads % kv_heads:
+            raise RuntimeError(f"attention: {heads} query heads over {kv_heads} key/value heads")
+        self.width, self.heads, self.kv_heads, self.dim, self.vdim, self.scale = width, heads, kv_heads, dim, vdim, float(scale)
+        self.dtype = torch.bfloat16
+
+    def input_parts(self, stc, prefix, dtype, device):
+        return [(self.tag + nm, _w(stc, prefix + nm, dtype, device), None) for nm in ("q", "k", "v")]
+
+    def load_rest(self, stc, prefix, dtype, device):
+        self.bias = _f32(stc, prefix + "pb", device)
+        self.w_o = _w(stc, prefix + "o", dtype, device)
+        assert self.bias.numel() == self.heads and self.w_o.shape == (self.width, self.heads * self.vdim)
+        self.dtype = dtype
+
+    def state_specs(self) -> list:
+        from .state_cache import PagedSpec
+        return [PagedSpec(self.tag + "k", (self.kv_heads * self.dim,), self.dtype), PagedSpec(self.tag + "v", (self.kv_heads * self.vdim,), self.dtype)]
+
+    def run(self, p: dict, inp: FusedInput, sb: StepBatch, state: dict) -> torch.Tensor:
+        H, G, d, dv, t = self.heads, self.kv_heads, self.dim, self.vdim, self.tag
+        q, k, v = p[t + "q"], p[t + "k"], p[t + "v"]
+        assert q.shape[1] == H * d and k.shape[1] == G * d and v.shape[1] == G * dv
+        kp, vp, table = state[t + "k"], state[t + "v"], state["page_table"]
+        mix_ops.paged_store(kp, vp, k, v, table, sb.tok_seq, sb.tok_pos, sb.slots)
+        out = torch.empty((sb.n, H * dv), dtype=self.dtype, device=q.device)
+        if sb.decode:
+            mix_ops.sigattn_decode(out, q, kp, vp, self.bias, table, sb.slots, sb.len_after, H, G, d, dv, self.scale)
+        else:
+            mix_ops.sigattn_prefill(out, q, k, v, self.bias, sb.cu, sb.tok_seq, H, G, d, dv, self.scale, sb.max_rows)
+        return F.linear(out, self.w_o)
+
+
+class MatrixLSTM(_SideMixer):
+    """mLSTM: q = W_q h dim^(-1/2), k, v per head; log gates i = cap tanh((W_i h + b_i) / cap), f = logsigmoid(cap tanh((W_f h + b_f) / cap)); running maximum
+    m' = max(f + m, i) (m = 0 at the start); S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise with k; o = S^T q / (max(|n.q|, e^(-m')) + 1e-6); per-head unit
+    RMS, a weight over all heads' values, sigmoid(W_g h), W_o.  State per slot: S [heads, vdim, dim], n [heads, dim], m [heads], float32."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, gate_cap: float, eps: float):
+        self.width, self.heads, self.dim, self.vdim, self.cap, self.eps = width, heads, dim, vdim, float(gate_cap), float(eps)
+        self.q_scale = float(dim) ** -0.5
+        self.dtype = torch.bfloat16
+
+    def input_parts(self, stc, prefix, dtype, device):
+        return [(self.tag + nm, _w(stc, prefix + nm, dtype, device), None) for nm in ("q", "k", "v", "g", "i", "f")]
+
+    def load_rest(self, stc, prefix, dtype, device):
+        self.bias_i, self.bias_f = _f32(stc, prefix + "i.b", device), _f32(stc, prefix + "f.b", device)
+        self.norm_w = _f32(stc, prefix + "norm", device)
+        self.w_o = _w(stc, prefix + "o", dtype, device)
+        assert self.norm_w.numel() == self.heads * self.vdim and self.w_o.shape == (self.width, self.heads * self.vdim) and self.bias_i.numel() == self.heads
+        self.dtype = dtype
+
+    def state_specs(self) -> list:
+        t = self.tag
+        return [StateSpec(t + "S", (self.heads, self.vdim, self.dim), torch.float32), StateSpec(t + "n", (self.heads, self.dim), torch.float32),
+                StateSpec(t + "m", (self.heads,), torch.float32)]
+
+    def run(self, p: dict, inp: FusedInput, sb: StepBatch, state: dict) -> torch.Tensor:
+        H, d, dv, t = self.heads, self.dim, self.vdim, self.tag
+        assert p[t + "q"].shape[1] == H * d and p[t + "v"].shape[1] == H * dv and p[t + "i"].shape[1] == H
+        o = torch.empty((sb.n, H, dv), dtype=torch.float32, device=self.w_o.device)
+        mix_ops.mlstm_scan(o, state[t + "S"], state[t + "n"], state[t + "m"], p[t + "q"], p[t + "k"], p[t + "v"], p[t + "i"], p[t + "f"], self.bias_i, self.bias_f,
+                           sb.cu, sb.slots, sb.pos0, self.q_scale, self.cap)
+        out = torch.empty((sb.n, H * dv), dtype=self.dtype, device=o.device)
+        mix_ops.head_norm_gate(out, o, self.norm_w, p[t + "g"], mix_ops.GATE_SIGMOID, self.eps)
+        return F.linear(out, self.w_o)
+
+
+class GatedDeltaRule(_SideMixer):
+    """Gated delta rule: q, k (kv_heads x dim) and v (heads x vdim) pass a short causal convolution per channel and silu; q, k become unit vectors per head
+    (x / sqrt(sum x^2 + 1e-6)), q times dim^(-1/2); beta = sigmoid(W_b h); decay g = exp(-exp(A_log) softplus(W_a h + dt_bias)) per head; per head S <- g S,
+    u = beta (v - S^T k), S <- S + k u^T, o = S^T q; per-head unit RMS, a weight over vdim shared by the heads, silu(W_g h), W_o.  State per slot: S
+    [heads, vdim, dim] float32 and the last taps - 1 rows of the projections q | k | v."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, taps: int, eps: float):
+        if heads % kv_heads:
+            raise RuntimeError(f"delta rule: {heads} value heads over {kv_heads} query/key heads")
+        if taps < 1 or taps > 16:
+            raise RuntimeError(f"delta rule: {taps} taps")
+        self.width, self.heads, self.kv_heads, self.dim, self.vdim, self.taps, self.eps = width, heads, kv_heads, dim, vdim, int(taps), float(eps)
+        self.channels = 2 * kv_heads * dim + heads * vdim
+        self.q_scale = float(dim) ** -0.5
+        self.dtype = torch.bfloat16
+
+    def input_parts(self, stc, prefix, dtype, device):
+        return [(self.tag + nm, _w(stc, prefix + nm, dtype, device), None) for nm in ("q", "k", "v", "b", "a", "g")]       # q, k, v side by side: one block
+
+    def load_rest(self, stc, prefix, dtype, device):
+        conv = torch.cat([_f32(stc, prefix + nm + ".conv", device) for nm in ("q", "k", "v")], dim=0)      # [channels, taps]
+        self.conv = conv.t().contiguous()
+        self.A_log, self.dt_bias = _f32(stc, prefix + "A_log", device), _f32(stc, prefix + "dt_bias", device)
+        self.norm_w = _f32(stc, prefix + "norm", device)
+        self.w_o = _w(stc, prefix + "o", dtype, device)
+        assert self.conv.shape == (self.taps, self.channels) and self.A_log.numel() == self.heads and self.norm_w.numel() == self.vdim
+        assert self.w_o.shape == (self.width, self.heads * self.vdim)
+        self.dtype = dtype
+
+    def state_specs(self) -> list:
+        t = self.tag
+        return [StateSpec(t + "S", (self.heads, self.vdim, self.dim), torch.float32), StateSpec(t + "conv", (max(self.taps - 1, 1), self.channels), self.dtype)]
+
+    def run(self, p: dict, inp: FusedInput, sb: StepBatch, state: dict) -> torch.Tensor:
+        H, G, d, dv, t = self.heads, self.kv_heads, self.dim, self.vdim, self.tag
+        x = inp.block(p, t + "q", t + "v")
+        assert x.shape[1] == self.channels and p[t + "b"].shape[1] == H and p[t + "g"].shape[1] == H * dv
+        dev, f32 = self.w_o.device, torch.float32
+        q, k = torch.empty((sb.n, G * d), dtype=f32, device=dev), torch.empty((sb.n, G * d), dtype=f32, device=dev)
+        v = torch.empty((sb.n, H * dv), dtype=f32, device=dev)
+        beta, decay = torch.empty((sb.n, H), dtype=f32, device=dev), torch.empty((sb.n, H), dtype=f32, device=dev)
+        mix_ops.delta_prep(q, k, v, beta, decay, x, self.conv, state[t + "conv"], p[t + "b"], p[t + "a"], self.A_log, self.dt_bias, sb.tok_seq, sb.tok_pos, sb.slots,
+                           sb.pos0, sb.len_after, H, G, d, dv, self.q_scale)
+        o = torch.empty((sb.n, H, dv), dtype=f32, device=dev)
+        mix_ops.delta_scan(o, state[t + "S"], q, k, v, beta, decay, sb.cu, sb.slots, sb.pos0, G)
+        out = torch.empty((sb.n, H * dv), dtype=self.dtype, device=dev)
+        mix_ops.head_norm_gate(out, o, self.norm_w, p[t + "g"], mix_ops.GATE_SILU, self.eps)
+        return F.linear(out, self.w_o)
+
+
+class ParallelMixer(_SideMixer):
+    """Two mixers side by side that read the same input: ONE fused input product for both, then
+    result = mean of the two outputs, each RMS-normed over the model width with its own plain weight."""
+
+    def __init__(self, width: int, left, right, eps: float):
+        self.width, self.left, self.right, self.eps = width, left, right, float(eps)
+        left.tag, right.tag = "left.", "right."
+
+    def input_parts(self, stc, prefix, dtype, device):
+        return self.left.input_parts(stc, prefix + "left.", dtype, device) + self.right.input_parts(stc, prefix + "right.", dtype, device)
+
+    def load_rest(self, stc, prefix, dtype, device):
+        self.left.load_rest(stc, prefix + "left.", dtype, device)
+        self.right.load_rest(stc, prefix + "right.", dtype, device)
+        self.w_left, self.w_right = _f32(stc, prefix + "left.out", device), _f32(stc, prefix + "right.out", device)
+        assert self.w_left.numel() == self.width and self.w_right.numel() == self.width
+        self.dtype = dtype
+
+    def state_specs(self) -> list:
+        return self.left.state_specs() + self.right.state_specs()
+
+    def run(self, p: dict, inp: FusedInput, sb: StepBatch, state: dict) -> torch.Tensor:
+        a = self.left.run(p, inp, sb, state)
+        b = self.right.run(p, inp, sb, state)
+        out = torch.empty((sb.n, self.width), dtype=self.dtype, device=a.device)
+        mix_ops.rms_pair(out, a, self.w_left, b, self.w_right, 0.5, self.eps)
+        return out
+
+
+class ParallelBlock:
+    """x <- x + m (mixer(h) + ff(hn)) with hn = norm(x) and h = hn + conv(hn): ONE norm per layer, the feed-forward reads the normed rows, the mixer their short
+    causal convolution; m is the residual factor.  The block is entered with (hn, h) already computed and leaves by computing the next block's pair: the
+    residual update (both sublayers' outputs, the factor, float32) and the next layer norm are one kernel."""
+
+    def __init__(self, width: int, eps: float, taps: int, mixer, mlp, residual_mult: float = 1.0):
+        self.width, self.eps, self.mixer, self.mlp, self.mult = width, float(eps), mixer, mlp, float(residual_mult)
+        self.in1 = LayerNormConv(width, taps, eps)
+
+    def load(self, stc, prefix: str, dtype, device):
+        self.in1.load(stc, prefix + "norm1", prefix + "canon1", dtype, device)
+        self.mixer.load(stc, prefix + "mix.", dtype, device)
+        if self.mlp is not None:
+            self.mlp.load(stc, prefix + "mlp.", dtype, device)
+        self.dtype = dtype
+
+    def state_specs(self) -> list:
+        return self.mixer.state_specs() + [self.in1.state_spec("canon1")]
+
+    def forward(self, x: torch.Tensor, hn: torch.Tensor, h: torch.Tensor, sb: StepBatch, state: dict, nxt: tuple | None):
+        """x: float32 residual (updated in place).  nxt = (the next block's LayerNormConv, its ring): returns the next block's (hn, h); None: the bare update."""
+        y, _ = self.mixer.forward(h, sb, state)
+        y2 = self.mlp.forward(hn, sb)[0] if self.mlp is not None else None
+        if nxt is None:
+            mix_ops.residual_norm_conv(x, y, y2, self.mult, mix_ops.RES_ADD, False, None, None, self.eps, None)
+            return None
+        return nxt[0].apply(x, y, y2, self.mult, mix_ops.RES_ADD, sb, nxt[1])

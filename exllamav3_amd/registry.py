@@ -3,7 +3,7 @@ Model registry: config.json names an architecture, the registry maps it to the c
 
     load_model(directory, device, dtype)  ->  a model with  .vocab, .new_cache(slots), .step(StepBatch, cache) -> float32 logits
 
-Registered: the unquantized mixer families (Vofanex, Zagilorn, Fimunex) with the step interface above, and the EXL3-quantized Llama of llama_path.py, which
+Registered: the unquantized mixer families (Vofanex, Zagilorn, Fimunex, Dikopel) with the step interface above, and the EXL3-quantized Llama of llama_path.py, which
 keeps its own decode_step / prefill_chunk pipelines (`load_model` returns it for `LlamaForCausalLM` checkpoints; the token-level
 generator drives step-interface models only).
 """
@@ -69,6 +69,12 @@ def _load_zagilorn(directory, config, device, dtype):
 def _load_fimunex(directory, config, device, dtype):
     from .fimunex import FimunexModel
     return FimunexModel.from_directory(directory, device=device, dtype=dtype or torch.bfloat16)
+
+
+@register("Dikopel", libraries=("mix",))
+def _load_dikopel(directory, config, device, dtype):
+    from .dikopel import DikopelModel
+    return DikopelModel.from_directory(directory, device=device, dtype=dtype or torch.bfloat16)
 
 
 @register("LlamaForCausalLM")

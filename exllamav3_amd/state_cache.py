@@ -5,6 +5,11 @@ float32 matrix per head for a recurrent (linear-attention) layer.  Slots are han
 and used again by the next one; the pool grows by doubling when every slot is taken.  Nothing in a slot has to be cleared on reuse: a
 mixer starts a sequence (position 0) from its own initial state and reads only what the sequence's length says is valid.
 
+A mixer whose memory grows with the sequence (attention without a window) declares `PagedSpec` buffers instead: per layer a POOL of pages of
+`page_size` tokens shared by all sequences, and one table [slots, pages per slot] that lists, in order, the pages a sequence owns (the same for every
+layer: they all hold the same tokens).  Pages are handed out as a sequence grows (in `begin_step`), given back with its slot and used again; the pool
+and the table grow by doubling.  Nothing is cleared: a reader takes the sequence's length from the step.
+
 `StepBatch` describes one step of the engine over these slots: the packed rows of all sequences in the step, and where each sequence
 stands.  The generator's scheduler and the trace runner both build it through `SlotStateCache.begin_step`.
 """
@@ -16,6 +21,14 @@ import torch
 @dataclass
 class StateSpec:
     """One per-slot buffer of a layer: name, shape per slot, element type."""
+    name: str
+    shape: tuple
+    dtype: torch.dtype
+
+
+@dataclass
+class PagedSpec:
+    """One per-token buffer of a layer, kept in pages: name, shape per token, element type.  The pool is [pages, page_size, *shape]."""
     name: str
     shape: tuple
     dtype: torch.dtype
@@ -40,15 +53,28 @@ class StepBatch:
 
 
 class SlotStateCache:
-    def __init__(self, layer_specs: list[list[StateSpec]], device, slots: int = 4):
+    def __init__(self, layer_specs: list[list], device, slots: int = 4, page_size: int = 64, tokens: int = 0):
+        """tokens: the most tokens that live sequences hold at once, if known -- sizes the page pools (they grow when it was too small)."""
         self.device = torch.device(device)
-        self.layer_specs = layer_specs
+        self.layer_specs = [[s for s in specs if isinstance(s, StateSpec)] for specs in layer_specs]
+        self.paged_specs = [[s for s in specs if isinstance(s, PagedSpec)] for specs in layer_specs]
         self.capacity = 0
         self.layers: list[dict[str, torch.Tensor]] = [dict() for _ in layer_specs]
         self.free: list[int] = []
         self.length: dict[int, int] = {}         # slot -> tokens held by the sequence that owns it
         self.generation = 0
+        self.paged = any(self.paged_specs)
+        self.page_size = int(page_size)
+        self.num_pages, self.free_pages, self.pages_of = 0, [], {}         # pages_of: slot -> its pages, in order
+        self.table_width = 0
+        self.page_table = self._table_host = None
         self._grow(max(1, slots))
+        if self.paged:
+            if self.page_size < 1:
+                raise RuntimeError("pages hold at least one token")
+            want = -(-int(tokens) // self.page_size) + max(1, slots) if tokens > 0 else 16
+            self._grow_table(max(1, -(-int(tokens) // self.page_size)) if tokens > 0 else 4)
+            self._grow_pages(want)
 
     def bytes_per_slot(self) -> int:
         total = 0
@@ -71,6 +97,60 @@ class SlotStateCache:
         self.free.extend(range(new_capacity - 1, self.capacity - 1, -1))      # lowest number on top of the stack
         self.capacity = new_capacity
         self.generation += 1                   # the buffers moved: whoever holds their addresses (captured graphs) starts over
+        if self.paged and self.table_width:
+            self._grow_table(self.table_width)
+
+    def _grow_table(self, width: int):
+        """The page table for `capacity` slots of `width` pages each (host copy + device copy; entries beyond a sequence's pages are 0 and never read)."""
+        host = torch.zeros((self.capacity, width), dtype=torch.int32)
+        if self._table_host is not None:
+            r, c = self._table_host.shape
+            host[:r, :c] = self._table_host
+        self._table_host, self.table_width = host, width
+        self.page_table = host.to(self.device)
+        for li, specs in enumerate(self.paged_specs):
+            if specs:
+                self.layers[li]["page_table"] = self.page_table
+        self.generation += 1
+
+    def _grow_pages(self, new_pages: int):
+        for li, specs in enumerate(self.paged_specs):
+            for s in specs:
+                buf = torch.zeros((new_pages, self.page_size) + tuple(s.shape), dtype=s.dtype, device=self.device)
+                old = self.layers[li].get(s.name)
+                if old is not None:
+                    buf[: self.num_pages].copy_(old)
+                self.layers[li][s.name] = buf
+        self.free_pages.extend(range(new_pages - 1, self.num_pages - 1, -1))
+        self.num_pages = new_pages
+        self.generation += 1
+
+    def reserve(self, entries: list[tuple[int, list[int]]]):
+        """Pages for the tokens that `entries` (slot, next tokens) are about to add.  begin_step calls it; a caller that holds device addresses (captured
+        graphs) calls it first and looks at `generation` afterwards."""
+        if not self.paged:
+            return
+        changed = []
+        for slot, toks in entries:
+            need = -(-(self.length[slot] + len(toks)) // self.page_size)
+            own = self.pages_of.setdefault(slot, [])
+            if need <= len(own):
+                continue
+            if need > self.table_width:
+                self._grow_table(max(need, 2 * self.table_width))
+            while len(own) < need:
+                if not self.free_pages:
+                    self._grow_pages(max(2 * self.num_pages, 1))
+                pg = self.free_pages.pop()
+                self._table_host[slot, len(own)] = pg
+                own.append(pg)
+            changed.append(slot)
+        if changed:
+            rows = torch.tensor(changed, dtype=torch.int64)
+            self.page_table.index_copy_(0, rows.to(self.device), self._table_host[rows].to(self.device))
+
+    def pages_in_use(self) -> int:
+        return self.num_pages - len(self.free_pages)
 
     def alloc(self) -> int:
         if not self.free:
@@ -84,6 +164,7 @@ class SlotStateCache:
             raise RuntimeError(f"slot {slot} is not in use")
         del self.length[slot]
         self.free.append(slot)
+        self.free_pages.extend(reversed(self.pages_of.pop(slot, [])))
 
     def in_use(self) -> int:
         return len(self.length)
@@ -100,6 +181,7 @@ class SlotStateCache:
         decode = all(l == 1 for l in lens) and any(p > 0 for p in pos0)
         if not decode and any(p > 0 for p in pos0):
             raise RuntimeError("a step either starts all its sequences or continues all of them by one token")
+        self.reserve(entries)
         n, b = sum(lens), len(entries)
         cu = [0]
         for l in lens:

@@ -15,9 +15,12 @@ import numpy as np
 
 
 class TraceSession:
-    def __init__(self, model, out_dir: str):
+    def __init__(self, model, out_dir: str, max_tokens: int = 0):
+        """max_tokens: the most tokens that live requests hold at once, if known: a model whose cache grows with its sequences sizes its pages from it."""
         self.model, self.out_dir = model, out_dir
-        self.cache = model.new_cache()
+        import inspect
+        sized = max_tokens > 0 and "tokens" in inspect.signature(model.new_cache).parameters
+        self.cache = model.new_cache(tokens=max_tokens) if sized else model.new_cache()
         self.slot_of: dict[str, int] = {}
 
     def run_step(self, rec: dict) -> int:

@@ -47,7 +47,7 @@ extern "C" {
 #define EXL3_MIX_MASK_WINDOW 0
 #define EXL3_MIX_MASK_CHUNK  1
 
-#define EXL3_MIX_ABI_VERSION 3
+#define EXL3_MIX_ABI_VERSION 4
 
 const char* exl3_mix_last_error(void);
 int  exl3_mix_abi_version(void);
@@ -278,6 +278,70 @@ int exl3_mix_moe_down_id(void* y, const void* hid, const void* wd, const int32_t
                          int n, int top, int experts, int ff, int width, int dtype, void* stream);
 int exl3_mix_moe_combine_id(void* y, const void* sorted, const int32_t* where, const float* wts, const int32_t* idx, int experts, const void* h_id,
                             const float* idw, int n, int top, int width, int dtype, void* stream);
+
+/* ---- parallel blocks over a layer norm, attention without softmax over paged keys, and recurrent mixers with a scalar decay per head ---- */
+
+/* x[n] = table[tokens[n]] * scale + P(tok_pos[n]); P: entry 2i = sin(p freq[i]), entry 2i + 1 = cos(p freq[i]) (float32 angles). */
+int exl3_mix_embed_sinusoid(float* x, const void* table, const int32_t* tokens, const int32_t* tok_pos, const float* freq, float scale, int n, int width, int vocab,
+                            int dtype, void* stream);
+
+/* h[i] = layer norm of residual row rows[i] (or i): (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b (b optional). */
+int exl3_mix_layer_norm_rows(void* h, const float* x, const int32_t* rows, const float* w, const float* b, float eps, int n, int width, int dtype, void* stream);
+
+/* The general form of exl3_mix_residual_rms.  mode 0: x stays; 1: x += y'; 2: x = y', with y' = (y + y2) * y_scale (y2 optional).  Then the norm of x:
+ * center 0: x / sqrt(mean(x^2) + eps) * w; center 1: the layer norm with weight w and optional bias.  hn_out (optional) receives the normed rows; h
+ * (optional) receives them too, or -- with conv_w [taps][width] and steps of one row per sequence -- normed row + its short causal convolution against
+ * the slot's ring of the last taps - 1 normed rows, which is updated. */
+int exl3_mix_residual_norm_conv(float* x, const void* y, int64_t y_ld, const void* y2, int64_t y2_ld, float y_scale, int mode, int center, const float* w,
+                                const float* bias, float eps, void* h, int64_t h_ld, void* hn_out, int64_t hn_ld, const float* conv_w, int taps, void* ring,
+                                const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots, int n, int width, int dtype, void* stream);
+
+/* exl3_mix_glu_act whose rows are also multiplied by sigmoid(rg[n]) (rg: one element per row, row stride rg_ld; may be null). */
+int exl3_mix_glu_act_rowgate(void* out, const void* g, int64_t g_ld, const void* u, int64_t u_ld, const void* rg, int64_t rg_ld, int n, int ff, int kind, float limit,
+                             int dtype, void* stream);
+
+/* exl3_mix_topk_grouped with a group's score = the sum of its group_top largest choice scores (1: its largest). */
+int exl3_mix_topk_grouped_ex(int32_t* idx, float* wts, float* idw, const float* logits, const float* correction, int kind, float scale, int normalise,
+                             int groups, int keep, int group_top, int n, int total, int real, int top, void* stream);
+
+/* Paged keys and values: pools k_pages [pages][page][kw], v_pages [pages][page][vw]; table [slots][table_ld] lists a sequence's pages in order.  Stores
+ * the step's rows (row n at position tok_pos[n] of sequence tok_seq[n]). */
+int exl3_mix_paged_store(void* k_pages, void* v_pages, const void* k, int64_t k_ld, const void* v, int64_t v_ld, const int32_t* table, int64_t table_ld, int page,
+                         const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots, int n, int kw, int vw, int dtype, void* stream);
+
+/* Causal attention without softmax: out[n][h] = sum over the keys j <= n of the row's sequence of sigmoid(scale q.k_j + bias[h]) v_j.  Prompt steps read
+ * the step's own keys (sequences start in the step); decode steps (one row per sequence) read the pages, len_after[n] keys. */
+int exl3_mix_sigattn_prefill(void* out, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v, int64_t v_ld, const float* bias,
+                             const int32_t* cu, const int32_t* tok_seq, int n, int heads, int kv_heads, int dim, int vdim, float scale, int dtype, void* stream);
+int exl3_mix_sigattn_decode(void* out, const void* q, int64_t q_ld, const void* k_pages, const void* v_pages, const float* bias, const int32_t* table, int64_t table_ld,
+                            int page, const int32_t* slots, const int32_t* len_after, int n, int heads, int kv_heads, int dim, int vdim, float scale, int dtype, void* stream);
+/* The same prompt step on the matrix cores (bfloat16; dim and vdim multiples of 16, dim <= 256, vdim <= 256). */
+int exl3_mix_sigattn_prefill_mfma(void* out, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v, int64_t v_ld, const float* bias,
+                                  const int32_t* cu, int batch, int max_rows, int heads, int kv_heads, int dim, int vdim, float scale, void* stream);
+
+/* mLSTM scan over the step's rows; state per slot: S [heads][vdim][dim], n [heads][dim], m [heads] (float32).  Sequences with pos0 == 0 start from zero
+ * (m = 0).  zi / zf: the gate projections (one per head), bias_i / bias_f their biases; log gates are capped: cap tanh(. / cap).  o [n][heads][vdim] float32. */
+int exl3_mix_mlstm_scan(float* o, float* S_state, float* n_state, float* m_state, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v, int64_t v_ld,
+                        const void* zi, int64_t zi_ld, const void* zf, int64_t zf_ld, const float* bias_i, const float* bias_f,
+                        const int32_t* cu, const int32_t* slots, const int32_t* pos0, int batch, int heads, int dim, int vdim, float q_scale, float cap,
+                        int dtype, void* stream);
+
+/* Gated delta rule: input stage (short convolutions with silu over x = q | k | v, unit query / key vectors, beta and decay; float32 results; ring
+ * [slots][taps - 1][C] of the last rows of x) and the scan (state S [slots][heads][vdim][dim] float32; query / key head = head / (heads / kv_heads)). */
+int exl3_mix_delta_prep(float* qo, float* ko, float* vo, float* beta, float* decay, const void* x, int64_t x_ld, const float* conv_w, int taps, void* ring,
+                        const void* zb, int64_t zb_ld, const void* za, int64_t za_ld, const float* A_log, const float* dt_bias,
+                        const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots, const int32_t* pos0, const int32_t* len_after,
+                        int n, int heads, int kv_heads, int dim, int vdim, float q_scale, int dtype, void* stream);
+int exl3_mix_delta_scan(float* o, float* S_state, const float* q, const float* k, const float* v, const float* beta, const float* decay,
+                        const int32_t* cu, const int32_t* slots, const int32_t* pos0, int batch, int heads, int kv_heads, int dim, int vdim, void* stream);
+
+/* out[n][h] = o[n][h] / rms(o[n][h]) * w[(per_head ? h vdim : 0) ..] * gate(g[n][h]); gate 0: silu, 1: sigmoid. */
+int exl3_mix_head_norm_gate(void* out, const float* o, const float* w, int per_head, const void* g, int64_t g_ld, int gate, float eps, int n, int heads, int vdim,
+                            int dtype, void* stream);
+
+/* out[n] = scale (a[n] / rms(a[n]) * wa + b[n] / rms(b[n]) * wb). */
+int exl3_mix_rms_pair(void* out, const void* a, int64_t a_ld, const float* wa, const void* b, int64_t b_ld, const float* wb, float scale, float eps, int n, int width,
+                      int dtype, void* stream);
 
 #ifdef __cplusplus
 }
