@@ -59,7 +59,9 @@ def parse():
                     help="instead of the default workload: layer times of the latent-attention family (Zagilorn) beside Vofanex layers of equal size, and its kernels' rooflines")
     ap.add_argument("--diff-family", action="store_true",
                     help="instead of the default workload: layer times of the differential-attention family (Fimunex) beside Vofanex layers of equal size, and its kernels' rooflines")
-    ap.add_argument("--mixer-sizes", default="", help="with --mixer-family / --latent-family / --diff-family: comma-separated sizes (1b, 8b; default both)")
+    ap.add_argument("--parallel-family", action="store_true",
+                    help="instead of the default workload: layer times of the parallel-block family (Dikopel) beside Vofanex layers of equal size, and its kernels' rooflines")
+    ap.add_argument("--mixer-sizes", default="", help="with --mixer-family / --latent-family / --diff-family / --parallel-family: comma-separated sizes (1b, 8b; default both)")
     ap.add_argument("--variant", type=int, default=1)
     ap.add_argument("--attention", action="store_true", help="include decode attention over the quantized KV cache (context = 1000 tokens) in the timed step")
     ap.add_argument("--unfused", action="store_true", help="one launch per reference op instead of the fused pipeline")
@@ -264,6 +266,9 @@ def main():
     if args.diff_family:
         from exllamav3_amd import diff_bench
         sys.exit(diff_bench.run(args))
+    if args.parallel_family:
+        from exllamav3_amd import parallel_bench
+        sys.exit(parallel_bench.run(args))
     import torch
     from exllamav3_amd import ext
     from exllamav3_amd.llama_path import SHAPES, SyntheticEXL3Llama
