@@ -6,12 +6,14 @@
 // Work split of the scans: one workgroup of 4 waves per (sequence, head, block of 16 value columns).  A wave owns 4 columns; the 16 lanes of a row
 // split the key channels of one column (lane kl holds channels kl, kl + 16, ... -- R of them, in registers), so that every product with the state is
 // R multiply-adds per lane and one sum over a row of 16 lanes (data-parallel primitives, no LDS).  The state is stored [slot][head][vdim][dim]: a row of
-// lanes reads consecutive floats.  A chunk of RC_TC tokens is staged in LDS; the waves run it without a barrier and the outputs leave through LDS.
+// lanes reads consecutive floats.  A chunk of 16 to 64 tokens is staged in LDS; the waves run it without a barrier and the outputs leave through LDS.
 // Everything that enters the recurrences is float32.
 #include "mix_common.cuh"
 
-#define RC_TC 16
 #define RC_COLS 16
+// tokens staged per chunk: as many as 32 KB of queries and keys allow.  A chunk pays one trip to memory, three barriers and the gates' transcendentals before its
+// token loop can start, and nothing overlaps them when a device holds fewer workgroups than it has compute units -- long chunks amortise that
+template <int R> struct rc_chunk { static constexpr int TC = R <= 4 ? 64 : (R <= 8 ? 32 : 16); };
 
 // ---------------------------------------------------------------------------------------------------------------------------------------------
 // mLSTM.  Per head and token, with log gates i (input) and f (forget) and the running maximum m (m = 0 before the first token):
@@ -25,8 +27,8 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(float* __restrict__ o, 
                                                          const int32_t* __restrict__ cu, const int32_t* __restrict__ slots, const int32_t* __restrict__ pos0,
                                                          int heads, int dim, int vdim, float q_scale, float cap)
 {
-    constexpr int DP = 16 * R;
-    __shared__ float qs[RC_TC * DP], ks[RC_TC * DP], vs[RC_TC * RC_COLS], gi[RC_TC], gf[RC_TC], os[RC_TC * RC_COLS];
+    constexpr int DP = 16 * R, RC_TC = rc_chunk<R>::TC;
+    __shared__ float qs[RC_TC * DP], ks[RC_TC * DP], vs[RC_TC * RC_COLS], gi[RC_TC], gf[RC_TC], sa[RC_TC], sb[RC_TC], se[RC_TC], os[RC_TC * RC_COLS], m_carry[2];
     const int b = blockIdx.x, h = blockIdx.y, vt = blockIdx.z;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int kl = lane & 15, cw = w * 4 + (lane >> 4);              // key lane, column inside the workgroup's block
@@ -45,23 +47,43 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(float* __restrict__ o, 
         S[r] = (resume && col_ok && c < dim) ? st[c] : 0.f;
         N[r] = (resume && c < dim) ? nst[c] : 0.f;
     }
-    float m = resume ? m_state[sh] : 0.f;
+    if (threadIdx.x == 0) m_carry[0] = resume ? m_state[sh] : 0.f;
+    int chunk = 0;
 
-    for (int n0 = first; n0 < last; n0 += RC_TC)
+    for (int n0 = first; n0 < last; n0 += RC_TC, ++chunk)
     {
         const int tc = min(RC_TC, last - n0);
+        const int tcp = (tc + 3) & ~3;                               // the token loop runs in groups of four; the tail is padded with tokens that change nothing
         __syncthreads();                                             // the previous chunk's LDS reads and output stores are over
-        for (int idx = threadIdx.x; idx < tc * DP; idx += 256)
+        // staging in batches of eight independent loads per thread: a loop that waits for every load in turn pays the trip to memory once per element
+        for (int base = threadIdx.x; base < tcp * DP; base += 256 * 8)
         {
-            const int t = idx / DP, c = idx - t * DP;
-            const int64_t n = n0 + t;
-            qs[idx] = c < dim ? to_f(q[n * q_ld + (int64_t) h * dim + c]) * q_scale : 0.f;
-            ks[idx] = c < dim ? to_f(k[n * k_ld + (int64_t) h * dim + c]) : 0.f;
+            float tq[8], tk[8];
+            #pragma unroll
+            for (int e = 0; e < 8; ++e)
+            {
+                const int idx = base + e * 256, t = idx / DP, c = idx - t * DP;
+                const bool ok = t < tc && c < dim;
+                tq[e] = ok ? to_f(q[(int64_t) (n0 + t) * q_ld + (int64_t) h * dim + c]) : 0.f;
+                tk[e] = ok ? to_f(k[(int64_t) (n0 + t) * k_ld + (int64_t) h * dim + c]) : 0.f;
+            }
+            #pragma unroll
+            for (int e = 0; e < 8; ++e)
+            {
+                const int idx = base + e * 256;
+                if (idx < tcp * DP) { qs[idx] = tq[e] * q_scale; ks[idx] = tk[e]; }
+            }
         }
-        for (int idx = threadIdx.x; idx < tc * RC_COLS; idx += 256)
         {
-            const int t = idx / RC_COLS, c = vt * RC_COLS + (idx - t * RC_COLS);
-            vs[idx] = c < vdim ? to_f(v[(int64_t) (n0 + t) * v_ld + (int64_t) h * vdim + c]) : 0.f;
+            float tv[RC_TC * RC_COLS / 256 > 0 ? RC_TC * RC_COLS / 256 : 1];
+            #pragma unroll
+            for (int e = 0; e < RC_TC * RC_COLS / 256; ++e)
+            {
+                const int idx = threadIdx.x + e * 256, t = idx / RC_COLS, c = vt * RC_COLS + (idx - t * RC_COLS);
+                tv[e] = (t < tc && c < vdim) ? to_f(v[(int64_t) (n0 + t) * v_ld + (int64_t) h * vdim + c]) : 0.f;
+            }
+            #pragma unroll
+            for (int e = 0; e < RC_TC * RC_COLS / 256; ++e) vs[threadIdx.x + e * 256] = tv[e];
         }
         if (threadIdx.x < tc)
         {
@@ -70,26 +92,42 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(float* __restrict__ o, 
             gf[threadIdx.x] = log_sigmoid_f(cap * tanhf((to_f(zf[n * zf_ld + h]) + bias_f[h]) / cap));
         }
         __syncthreads();
-        for (int t = 0; t < tc; ++t)
+        // The gates' part of the recurrence off the token loop: thread t walks the running maximum up to its token (an add and a max per token), then the three
+        // exponentials of all tokens are taken side by side.
+        if (threadIdx.x < tcp)
         {
-            const float f = gf[t], i = gi[t];
-            const float m_new = fmaxf(f + m, i);
-            const float a = expf(f + m - m_new), bb = expf(i - m_new);
-            m = m_new;
-            const float vv = vs[t * RC_COLS + cw] * bb;
-            float po = 0.f, pn = 0.f;
+            const int t = threadIdx.x;
+            float m = m_carry[chunk & 1], m_prev = m;
+            for (int u = 0; u <= t && u < tc; ++u) { m_prev = m; m = fmaxf(gf[u] + m, gi[u]); }
+            const bool real = t < tc;
+            sa[t] = real ? expf(gf[t] + m_prev - m) : 1.0f;
+            sb[t] = real ? expf(gi[t] - m) : 0.0f;
+            se[t] = expf(-m);
+            if (t == tc - 1) m_carry[(chunk + 1) & 1] = m;
+        }
+        __syncthreads();
+        for (int t0 = 0; t0 < tcp; t0 += 4)
+        {
             #pragma unroll
-            for (int r = 0; r < R; ++r)
+            for (int u = 0; u < 4; ++u)
             {
-                const float kk = ks[t * DP + kl + 16 * r], qq = qs[t * DP + kl + 16 * r];
-                S[r] = a * S[r] + kk * vv;
-                N[r] = a * N[r] + bb * kk;
-                po += qq * S[r];
-                pn += qq * N[r];
+                const int t = t0 + u;
+                const float a = sa[t], bb = sb[t];
+                const float vv = vs[t * RC_COLS + cw] * bb;
+                float po = 0.f, pn = 0.f;
+                #pragma unroll
+                for (int r = 0; r < R; ++r)
+                {
+                    const float kk = ks[t * DP + kl + 16 * r], qq = qs[t * DP + kl + 16 * r];
+                    S[r] = __builtin_fmaf(a, S[r], kk * vv);
+                    N[r] = __builtin_fmaf(a, N[r], bb * kk);
+                    po = __builtin_fmaf(qq, S[r], po);
+                    pn = __builtin_fmaf(qq, N[r], pn);
+                }
+                po = row16_sum(po);
+                pn = row16_sum(pn);
+                if (kl == 0) os[t * RC_COLS + cw] = po * __builtin_amdgcn_rcpf(fmaxf(fabsf(pn), se[t]) + 1e-6f);
             }
-            po = row16_sum(po);
-            pn = row16_sum(pn);
-            if (kl == 0) os[t * RC_COLS + cw] = po / (fmaxf(fabsf(pn), expf(-m)) + 1e-6f);
         }
         __syncthreads();
         for (int idx = threadIdx.x; idx < tc * RC_COLS; idx += 256)
@@ -105,7 +143,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(float* __restrict__ o, 
         if (col_ok && c < dim) st[c] = S[r];
         if (vt == 0 && cw == 0 && c < dim) nst[c] = N[r];
     }
-    if (vt == 0 && threadIdx.x == 0) m_state[sh] = m;
+    if (vt == 0 && threadIdx.x == 0) m_state[sh] = m_carry[chunk & 1];       // written by a thread of this workgroup before the last barrier
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------------------------
@@ -118,7 +156,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
                                                          const int32_t* __restrict__ cu, const int32_t* __restrict__ slots, const int32_t* __restrict__ pos0,
                                                          int heads, int kv_heads, int dim, int vdim)
 {
-    constexpr int DP = 16 * R;
+    constexpr int DP = 16 * R, RC_TC = rc_chunk<R>::TC;
     __shared__ float qs[RC_TC * DP], ks[RC_TC * DP], vs[RC_TC * RC_COLS], gs[RC_TC], bs[RC_TC], os[RC_TC * RC_COLS];
     const int b = blockIdx.x, h = blockIdx.y, vt = blockIdx.z;
     const int g = h / (heads / kv_heads);
@@ -140,46 +178,71 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
     for (int n0 = first; n0 < last; n0 += RC_TC)
     {
         const int tc = min(RC_TC, last - n0);
+        const int tcp = (tc + 3) & ~3;                               // groups of four tokens; the tail is padded with tokens that change nothing (g = 1, beta = 0)
         __syncthreads();
-        for (int idx = threadIdx.x; idx < tc * DP; idx += 256)
+        for (int base = threadIdx.x; base < tcp * DP; base += 256 * 8)          // eight independent loads per thread and batch (see mlstm_scan_kernel)
         {
-            const int t = idx / DP, c = idx - t * DP;
-            const int64_t at = (int64_t) (n0 + t) * qk_ld + (int64_t) g * dim + c;
-            qs[idx] = c < dim ? q[at] : 0.f;
-            ks[idx] = c < dim ? k[at] : 0.f;
-        }
-        for (int idx = threadIdx.x; idx < tc * RC_COLS; idx += 256)
-        {
-            const int t = idx / RC_COLS, c = vt * RC_COLS + (idx - t * RC_COLS);
-            vs[idx] = c < vdim ? v[((int64_t) (n0 + t) * heads + h) * vdim + c] : 0.f;
-        }
-        if (threadIdx.x < tc)
-        {
-            gs[threadIdx.x] = decay[(int64_t) (n0 + threadIdx.x) * heads + h];
-            bs[threadIdx.x] = beta[(int64_t) (n0 + threadIdx.x) * heads + h];
-        }
-        __syncthreads();
-        for (int t = 0; t < tc; ++t)
-        {
-            const float gg = gs[t], bb = bs[t], vv = vs[t * RC_COLS + cw];
-            float kk[R];
-            float pk = 0.f, pq = 0.f, qk = 0.f;
+            float tq[8], tk[8];
             #pragma unroll
-            for (int r = 0; r < R; ++r)
+            for (int e = 0; e < 8; ++e)
             {
-                kk[r] = ks[t * DP + kl + 16 * r];
-                const float qq = qs[t * DP + kl + 16 * r];
-                pk += kk[r] * S[r];
-                pq += qq * S[r];
-                qk += qq * kk[r];
+                const int idx = base + e * 256, t = idx / DP, c = idx - t * DP;
+                const int64_t at = (int64_t) (n0 + t) * qk_ld + (int64_t) g * dim + c;
+                const bool ok = t < tc && c < dim;
+                tq[e] = ok ? q[at] : 0.f;
+                tk[e] = ok ? k[at] : 0.f;
             }
-            pk = row16_sum(pk);
-            pq = row16_sum(pq);
-            qk = row16_sum(qk);
-            const float u = bb * (vv - gg * pk);
             #pragma unroll
-            for (int r = 0; r < R; ++r) S[r] = gg * S[r] + kk[r] * u;
-            if (kl == 0) os[t * RC_COLS + cw] = gg * pq + qk * u;
+            for (int e = 0; e < 8; ++e)
+            {
+                const int idx = base + e * 256;
+                if (idx < tcp * DP) { qs[idx] = tq[e]; ks[idx] = tk[e]; }
+            }
+        }
+        {
+            float tv[RC_TC * RC_COLS / 256 > 0 ? RC_TC * RC_COLS / 256 : 1];
+            #pragma unroll
+            for (int e = 0; e < RC_TC * RC_COLS / 256; ++e)
+            {
+                const int idx = threadIdx.x + e * 256, t = idx / RC_COLS, c = vt * RC_COLS + (idx - t * RC_COLS);
+                tv[e] = (t < tc && c < vdim) ? v[((int64_t) (n0 + t) * heads + h) * vdim + c] : 0.f;
+            }
+            #pragma unroll
+            for (int e = 0; e < RC_TC * RC_COLS / 256; ++e) vs[threadIdx.x + e * 256] = tv[e];
+        }
+        if (threadIdx.x < tcp)
+        {
+            const bool real = threadIdx.x < tc;
+            gs[threadIdx.x] = real ? decay[(int64_t) (n0 + threadIdx.x) * heads + h] : 1.0f;
+            bs[threadIdx.x] = real ? beta[(int64_t) (n0 + threadIdx.x) * heads + h] : 0.0f;
+        }
+        __syncthreads();
+        for (int t0 = 0; t0 < tcp; t0 += 4)
+        {
+            #pragma unroll
+            for (int u4 = 0; u4 < 4; ++u4)
+            {
+                const int t = t0 + u4;
+                const float gg = gs[t], bb = bs[t], vv = vs[t * RC_COLS + cw];
+                float kk[R];
+                float pk = 0.f, pk2 = 0.f, pq = 0.f, qk = 0.f;
+                #pragma unroll
+                for (int r = 0; r < R; ++r)
+                {
+                    kk[r] = ks[t * DP + kl + 16 * r];
+                    const float qq = qs[t * DP + kl + 16 * r];
+                    if (r & 1) pk2 = __builtin_fmaf(kk[r], S[r], pk2); else pk = __builtin_fmaf(kk[r], S[r], pk);      // the sum the next state waits for: two chains
+                    pq = __builtin_fmaf(qq, S[r], pq);
+                    qk = __builtin_fmaf(qq, kk[r], qk);
+                }
+                pk = row16_sum(pk + pk2);
+                const float u = bb * __builtin_fmaf(-gg, pk, vv);
+                #pragma unroll
+                for (int r = 0; r < R; ++r) S[r] = __builtin_fmaf(kk[r], u, gg * S[r]);
+                pq = row16_sum(pq);
+                qk = row16_sum(qk);
+                if (kl == 0) os[t * RC_COLS + cw] = __builtin_fmaf(qk, u, gg * pq);
+            }
         }
         __syncthreads();
         for (int idx = threadIdx.x; idx < tc * RC_COLS; idx += 256)
