@@ -11,14 +11,20 @@
 #include "mix_common.cuh"
 
 #define RC_COLS 16
-// tokens staged per chunk: as many as 32 KB of queries and keys allow.  A chunk pays one trip to memory, three barriers and the gates' transcendentals before its
-// token loop can start, and nothing overlaps them when a device holds fewer workgroups than it has compute units -- long chunks amortise that
+// tokens staged per chunk: as many as 32 KB of queries and keys allow (a chunk costs two barriers and, for mLSTM, the gates' transcendentals)
 template <int R> struct rc_chunk { static constexpr int TC = R <= 4 ? 64 : (R <= 8 ? 32 : 16); };
 
 // ---------------------------------------------------------------------------------------------------------------------------------------------
+// How both scans walk a sequence.  The rows of chunk c + 1 are loaded into REGISTERS before the token loop of chunk c starts and stored to LDS after it ends, so
+// the trip to memory runs under the token loop (with fewer workgroups than compute units nothing else would hide it).  Per chunk: registers -> LDS, barrier,
+// loads of the next chunk, token loop in groups of four (the tail of a chunk is padded with tokens that change nothing), barrier, outputs from LDS to memory.
+
 // mLSTM.  Per head and token, with log gates i (input) and f (forget) and the running maximum m (m = 0 before the first token):
 //   m' = max(f + m, i);  a = exp(f + m - m'), b = exp(i - m');  S <- a S + b k v^T;  n <- a n + b k;  o = S^T q / (max(|n.q|, exp(-m')) + 1e-6)
 // i = cap tanh((z_i + bias_i) / cap), f = logsigmoid(cap tanh((z_f + bias_f) / cap)) from the projections z_i, z_f.  q is scaled by q_scale.
+// The gates' part of the recurrence stays off the token loop: a token is the map m -> max(m + f, i), maps compose to maps of the same form
+// ((f1, i1) then (f2, i2) = (f1 + f2, max(i1 + f2, i2))), so one wave scans a chunk's maps across its lanes in six steps and takes the exponentials of all
+// tokens side by side.
 template <typename T, int R>
 __global__ __launch_bounds__(256) void mlstm_scan_kernel(float* __restrict__ o, float* __restrict__ S_state, float* __restrict__ n_state, float* __restrict__ m_state,
                                                          const T* __restrict__ q, int64_t q_ld, const T* __restrict__ k, int64_t k_ld, const T* __restrict__ v, int64_t v_ld,
@@ -27,8 +33,8 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(float* __restrict__ o, 
                                                          const int32_t* __restrict__ cu, const int32_t* __restrict__ slots, const int32_t* __restrict__ pos0,
                                                          int heads, int dim, int vdim, float q_scale, float cap)
 {
-    constexpr int DP = 16 * R, RC_TC = rc_chunk<R>::TC;
-    __shared__ float qs[RC_TC * DP], ks[RC_TC * DP], vs[RC_TC * RC_COLS], gi[RC_TC], gf[RC_TC], sa[RC_TC], sb[RC_TC], se[RC_TC], os[RC_TC * RC_COLS], m_carry[2];
+    constexpr int DP = 16 * R, RC_TC = rc_chunk<R>::TC, NPT = RC_TC * DP / 256, NVT = RC_TC * RC_COLS / 256;
+    __shared__ __attribute__((aligned(16))) float qs[RC_TC * DP], ks[RC_TC * DP], vs[RC_TC * RC_COLS], sa[RC_TC], sb[RC_TC], se[RC_TC], os[RC_TC * RC_COLS];
     const int b = blockIdx.x, h = blockIdx.y, vt = blockIdx.z;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int kl = lane & 15, cw = w * 4 + (lane >> 4);              // key lane, column inside the workgroup's block
@@ -47,65 +53,72 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(float* __restrict__ o, 
         S[r] = (resume && col_ok && c < dim) ? st[c] : 0.f;
         N[r] = (resume && c < dim) ? nst[c] : 0.f;
     }
-    if (threadIdx.x == 0) m_carry[0] = resume ? m_state[sh] : 0.f;
-    int chunk = 0;
+    float m_run = resume ? m_state[sh] : 0.f;                        // kept current by wave 0
+    const float bi = bias_i[h], bfg = bias_f[h];
+    T tq[NPT], tk[NPT], tv[NVT], tzi = from_f<T>(0.f), tzf = from_f<T>(0.f);      // held as loaded: a conversion here would wait for the loads before the token loop
+    const T zero = from_f<T>(0.f);
+    #define ML_FETCH(N0) \
+        do { \
+            const int f_tc = min(RC_TC, last - (N0)); \
+            _Pragma("unroll") \
+            for (int e = 0; e < NPT; ++e) \
+            { \
+                const int idx = threadIdx.x + e * 256, t = idx / DP, c = idx - t * DP; \
+                const bool ok = t < f_tc && c < dim; \
+                tq[e] = ok ? q[(int64_t) ((N0) + t) * q_ld + (int64_t) h * dim + c] : zero; \
+                tk[e] = ok ? k[(int64_t) ((N0) + t) * k_ld + (int64_t) h * dim + c] : zero; \
+            } \
+            _Pragma("unroll") \
+            for (int e = 0; e < NVT; ++e) \
+            { \
+                const int idx = threadIdx.x + e * 256, t = idx / RC_COLS, c = vt * RC_COLS + (idx - t * RC_COLS); \
+                tv[e] = (t < f_tc && c < vdim) ? v[(int64_t) ((N0) + t) * v_ld + (int64_t) h * vdim + c] : zero; \
+            } \
+            if (w == 0 && lane < f_tc) \
+            { \
+                tzi = zi[(int64_t) ((N0) + lane) * zi_ld + h]; \
+                tzf = zf[(int64_t) ((N0) + lane) * zf_ld + h]; \
+            } \
+        } while (0)
+    if (first < last) ML_FETCH(first);
 
-    for (int n0 = first; n0 < last; n0 += RC_TC, ++chunk)
+    for (int n0 = first; n0 < last; n0 += RC_TC)
     {
         const int tc = min(RC_TC, last - n0);
-        const int tcp = (tc + 3) & ~3;                               // the token loop runs in groups of four; the tail is padded with tokens that change nothing
-        __syncthreads();                                             // the previous chunk's LDS reads and output stores are over
-        // staging in batches of eight independent loads per thread: a loop that waits for every load in turn pays the trip to memory once per element
-        for (int base = threadIdx.x; base < tcp * DP; base += 256 * 8)
+        const int tcp = (tc + 3) & ~3;
+        #pragma unroll
+        for (int e = 0; e < NPT; ++e)
         {
-            float tq[8], tk[8];
-            #pragma unroll
-            for (int e = 0; e < 8; ++e)
-            {
-                const int idx = base + e * 256, t = idx / DP, c = idx - t * DP;
-                const bool ok = t < tc && c < dim;
-                tq[e] = ok ? to_f(q[(int64_t) (n0 + t) * q_ld + (int64_t) h * dim + c]) : 0.f;
-                tk[e] = ok ? to_f(k[(int64_t) (n0 + t) * k_ld + (int64_t) h * dim + c]) : 0.f;
-            }
-            #pragma unroll
-            for (int e = 0; e < 8; ++e)
-            {
-                const int idx = base + e * 256;
-                if (idx < tcp * DP) { qs[idx] = tq[e] * q_scale; ks[idx] = tk[e]; }
-            }
+            const int idx = threadIdx.x + e * 256, t = idx / DP, c = idx - t * DP, at = t * DP + (c & 15) * R + (c >> 4);      // a lane's R channels side by side
+            qs[at] = to_f(tq[e]) * q_scale; ks[at] = to_f(tk[e]);
         }
+        #pragma unroll
+        for (int e = 0; e < NVT; ++e) vs[threadIdx.x + e * 256] = to_f(tv[e]);
+        if (w == 0)
         {
-            float tv[RC_TC * RC_COLS / 256 > 0 ? RC_TC * RC_COLS / 256 : 1];
+            const bool real = lane < tc;
+            const float F = real ? log_sigmoid_f(cap * tanhf((to_f(tzf) + bfg) / cap)) : 0.f;
+            const float I = real ? cap * tanhf((to_f(tzi) + bi) / cap) : -INFINITY;
+            float sF = F, sM = I;                                    // the composition of the chunk's maps up to this lane's token
             #pragma unroll
-            for (int e = 0; e < RC_TC * RC_COLS / 256; ++e)
+            for (int off = 1; off < 64; off <<= 1)
             {
-                const int idx = threadIdx.x + e * 256, t = idx / RC_COLS, c = vt * RC_COLS + (idx - t * RC_COLS);
-                tv[e] = (t < tc && c < vdim) ? to_f(v[(int64_t) (n0 + t) * v_ld + (int64_t) h * vdim + c]) : 0.f;
+                const float pF = __shfl_up(sF, off, 64), pM = __shfl_up(sM, off, 64);
+                if (lane >= off) { sM = fmaxf(pM + sF, sM); sF = pF + sF; }
             }
-            #pragma unroll
-            for (int e = 0; e < RC_TC * RC_COLS / 256; ++e) vs[threadIdx.x + e * 256] = tv[e];
-        }
-        if (threadIdx.x < tc)
-        {
-            const int64_t n = n0 + threadIdx.x;
-            gi[threadIdx.x] = cap * tanhf((to_f(zi[n * zi_ld + h]) + bias_i[h]) / cap);
-            gf[threadIdx.x] = log_sigmoid_f(cap * tanhf((to_f(zf[n * zf_ld + h]) + bias_f[h]) / cap));
+            const float m_t = fmaxf(m_run + sF, sM);
+            float m_prev = __shfl_up(m_t, 1, 64);
+            if (lane == 0) m_prev = m_run;
+            if (lane < RC_TC)
+            {
+                sa[lane] = real ? expf(F + m_prev - m_t) : 1.0f;
+                sb[lane] = real ? expf(I - m_t) : 0.0f;
+                se[lane] = expf(-m_t);
+            }
+            m_run = __shfl(m_t, tc - 1, 64);
         }
         __syncthreads();
-        // The gates' part of the recurrence off the token loop: thread t walks the running maximum up to its token (an add and a max per token), then the three
-        // exponentials of all tokens are taken side by side.
-        if (threadIdx.x < tcp)
-        {
-            const int t = threadIdx.x;
-            float m = m_carry[chunk & 1], m_prev = m;
-            for (int u = 0; u <= t && u < tc; ++u) { m_prev = m; m = fmaxf(gf[u] + m, gi[u]); }
-            const bool real = t < tc;
-            sa[t] = real ? expf(gf[t] + m_prev - m) : 1.0f;
-            sb[t] = real ? expf(gi[t] - m) : 0.0f;
-            se[t] = expf(-m);
-            if (t == tc - 1) m_carry[(chunk + 1) & 1] = m;
-        }
-        __syncthreads();
+        if (n0 + RC_TC < last) ML_FETCH(n0 + RC_TC);                 // in flight during the token loop
         for (int t0 = 0; t0 < tcp; t0 += 4)
         {
             #pragma unroll
@@ -118,7 +131,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(float* __restrict__ o, 
                 #pragma unroll
                 for (int r = 0; r < R; ++r)
                 {
-                    const float kk = ks[t * DP + kl + 16 * r], qq = qs[t * DP + kl + 16 * r];
+                    const float kk = ks[t * DP + kl * R + r], qq = qs[t * DP + kl * R + r];
                     S[r] = __builtin_fmaf(a, S[r], kk * vv);
                     N[r] = __builtin_fmaf(a, N[r], bb * kk);
                     po = __builtin_fmaf(qq, S[r], po);
@@ -136,6 +149,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(float* __restrict__ o, 
             if (c < vdim) o[((int64_t) (n0 + t) * heads + h) * vdim + c] = os[idx];
         }
     }
+    #undef ML_FETCH
     #pragma unroll
     for (int r = 0; r < R; ++r)
     {
@@ -143,7 +157,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(float* __restrict__ o, 
         if (col_ok && c < dim) st[c] = S[r];
         if (vt == 0 && cw == 0 && c < dim) nst[c] = N[r];
     }
-    if (vt == 0 && threadIdx.x == 0) m_state[sh] = m_carry[chunk & 1];       // written by a thread of this workgroup before the last barrier
+    if (vt == 0 && threadIdx.x == 0) m_state[sh] = m_run;
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------------------------
@@ -156,8 +170,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
                                                          const int32_t* __restrict__ cu, const int32_t* __restrict__ slots, const int32_t* __restrict__ pos0,
                                                          int heads, int kv_heads, int dim, int vdim)
 {
-    constexpr int DP = 16 * R, RC_TC = rc_chunk<R>::TC;
-    __shared__ float qs[RC_TC * DP], ks[RC_TC * DP], vs[RC_TC * RC_COLS], gs[RC_TC], bs[RC_TC], os[RC_TC * RC_COLS];
+    constexpr int DP = 16 * R, RC_TC = rc_chunk<R>::TC, NPT = RC_TC * DP / 256, NVT = RC_TC * RC_COLS / 256;
+    __shared__ __attribute__((aligned(16))) float qs[RC_TC * DP], ks[RC_TC * DP], vs[RC_TC * RC_COLS], gs[RC_TC], bs[RC_TC], os[RC_TC * RC_COLS];
     const int b = blockIdx.x, h = blockIdx.y, vt = blockIdx.z;
     const int g = h / (heads / kv_heads);
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -175,48 +189,46 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
         const int c = kl + 16 * r;
         S[r] = (resume && col_ok && c < dim) ? st[c] : 0.f;
     }
+    float tq[NPT], tk[NPT], tv[NVT], tg = 1.0f, tb = 0.0f;
+    #define DL_FETCH(N0) \
+        do { \
+            const int f_tc = min(RC_TC, last - (N0)); \
+            _Pragma("unroll") \
+            for (int e = 0; e < NPT; ++e) \
+            { \
+                const int idx = threadIdx.x + e * 256, t = idx / DP, c = idx - t * DP; \
+                const int64_t at = (int64_t) ((N0) + t) * qk_ld + (int64_t) g * dim + c; \
+                const bool ok = t < f_tc && c < dim; \
+                tq[e] = ok ? q[at] : 0.f; \
+                tk[e] = ok ? k[at] : 0.f; \
+            } \
+            _Pragma("unroll") \
+            for (int e = 0; e < NVT; ++e) \
+            { \
+                const int idx = threadIdx.x + e * 256, t = idx / RC_COLS, c = vt * RC_COLS + (idx - t * RC_COLS); \
+                tv[e] = (t < f_tc && c < vdim) ? v[((int64_t) ((N0) + t) * heads + h) * vdim + c] : 0.f; \
+            } \
+            const bool f_real = (int) threadIdx.x < f_tc;            /* padding: g = 1, beta = 0 */ \
+            tg = f_real ? decay[(int64_t) ((N0) + threadIdx.x) * heads + h] : 1.0f; \
+            tb = f_real ? beta[(int64_t) ((N0) + threadIdx.x) * heads + h] : 0.0f; \
+        } while (0)
+    if (first < last) DL_FETCH(first);
+
     for (int n0 = first; n0 < last; n0 += RC_TC)
     {
         const int tc = min(RC_TC, last - n0);
-        const int tcp = (tc + 3) & ~3;                               // groups of four tokens; the tail is padded with tokens that change nothing (g = 1, beta = 0)
+        const int tcp = (tc + 3) & ~3;
+        #pragma unroll
+        for (int e = 0; e < NPT; ++e)
+        {
+            const int idx = threadIdx.x + e * 256, t = idx / DP, c = idx - t * DP, at = t * DP + (c & 15) * R + (c >> 4);      // a lane's R channels side by side
+            qs[at] = tq[e]; ks[at] = tk[e];
+        }
+        #pragma unroll
+        for (int e = 0; e < NVT; ++e) vs[threadIdx.x + e * 256] = tv[e];
+        if (threadIdx.x < RC_TC) { gs[threadIdx.x] = tg; bs[threadIdx.x] = tb; }
         __syncthreads();
-        for (int base = threadIdx.x; base < tcp * DP; base += 256 * 8)          // eight independent loads per thread and batch (see mlstm_scan_kernel)
-        {
-            float tq[8], tk[8];
-            #pragma unroll
-            for (int e = 0; e < 8; ++e)
-            {
-                const int idx = base + e * 256, t = idx / DP, c = idx - t * DP;
-                const int64_t at = (int64_t) (n0 + t) * qk_ld + (int64_t) g * dim + c;
-                const bool ok = t < tc && c < dim;
-                tq[e] = ok ? q[at] : 0.f;
-                tk[e] = ok ? k[at] : 0.f;
-            }
-            #pragma unroll
-            for (int e = 0; e < 8; ++e)
-            {
-                const int idx = base + e * 256;
-                if (idx < tcp * DP) { qs[idx] = tq[e]; ks[idx] = tk[e]; }
-            }
-        }
-        {
-            float tv[RC_TC * RC_COLS / 256 > 0 ? RC_TC * RC_COLS / 256 : 1];
-            #pragma unroll
-            for (int e = 0; e < RC_TC * RC_COLS / 256; ++e)
-            {
-                const int idx = threadIdx.x + e * 256, t = idx / RC_COLS, c = vt * RC_COLS + (idx - t * RC_COLS);
-                tv[e] = (t < tc && c < vdim) ? v[((int64_t) (n0 + t) * heads + h) * vdim + c] : 0.f;
-            }
-            #pragma unroll
-            for (int e = 0; e < RC_TC * RC_COLS / 256; ++e) vs[threadIdx.x + e * 256] = tv[e];
-        }
-        if (threadIdx.x < tcp)
-        {
-            const bool real = threadIdx.x < tc;
-            gs[threadIdx.x] = real ? decay[(int64_t) (n0 + threadIdx.x) * heads + h] : 1.0f;
-            bs[threadIdx.x] = real ? beta[(int64_t) (n0 + threadIdx.x) * heads + h] : 0.0f;
-        }
-        __syncthreads();
+        if (n0 + RC_TC < last) DL_FETCH(n0 + RC_TC);                 // in flight during the token loop
         for (int t0 = 0; t0 < tcp; t0 += 4)
         {
             #pragma unroll
@@ -229,8 +241,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
                 #pragma unroll
                 for (int r = 0; r < R; ++r)
                 {
-                    kk[r] = ks[t * DP + kl + 16 * r];
-                    const float qq = qs[t * DP + kl + 16 * r];
+                    kk[r] = ks[t * DP + kl * R + r];
+                    const float qq = qs[t * DP + kl * R + r];
                     if (r & 1) pk2 = __builtin_fmaf(kk[r], S[r], pk2); else pk = __builtin_fmaf(kk[r], S[r], pk);      // the sum the next state waits for: two chains
                     pq = __builtin_fmaf(qq, S[r], pq);
                     qk = __builtin_fmaf(qq, kk[r], qk);
@@ -251,6 +263,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
             if (c < vdim) o[((int64_t) (n0 + t) * heads + h) * vdim + c] = os[idx];
         }
     }
+    #undef DL_FETCH
     #pragma unroll
     for (int r = 0; r < R; ++r)
     {
