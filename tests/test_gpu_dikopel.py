@@ -443,7 +443,7 @@ def test_mlstm_scan_prompt_then_decode(gpu, dtype, H, d, dv, cap):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,d,dv,taps", [(4, 2, 16, 8, 4), (2, 2, 8, 12, 1), (6, 1, 20, 6, 2), (2, 1, 128, 64, 3), (1, 1, 40, 100, 3)])
+@pytest.mark.parametrize("H,G,d,dv,taps", [(4, 2, 16, 8, 4), (2, 2, 8, 12, 1), (6, 1, 20, 6, 2), (2, 1, 128, 64, 3), (1, 1, 40, 100, 3), (2, 1, 200, 24, 2)])
 def test_gated_delta_rule_prompt_then_decode(gpu, dtype, H, G, d, dv, taps):
     """Input stage (short convolutions with silu, unit vectors, step size, decay) and scan against the oracle's token loop, then decoding from the slots: the
     convolution's predecessors then come from the slot's ring, the state from the slot."""
